@@ -1,6 +1,7 @@
 from .model_config import ConfigError, LlamaConfig, RopeScaling, read_config_json
 from .feduzen_config import FeduzenConfig
 from .mogisun_config import MogisunConfig
+from .famepel_config import FamepelConfig
 from .engine_config import EngineConfig, resolve_dtype
 from .registry import (
     Architecture, UnknownArchitecture, architecture_name, architecture_of, get_architecture,
@@ -9,7 +10,7 @@ from .registry import (
 from .presets import PRESETS, preset
 
 __all__ = [
-    "ConfigError", "FeduzenConfig", "LlamaConfig", "MogisunConfig", "RopeScaling", "read_config_json",
+    "ConfigError", "FamepelConfig", "FeduzenConfig", "LlamaConfig", "MogisunConfig", "RopeScaling", "read_config_json",
     "EngineConfig", "resolve_dtype",
     "Architecture", "UnknownArchitecture", "architecture_name", "architecture_of", "get_architecture",
     "known_architectures", "register_architecture", "unregister_architecture",

@@ -5,7 +5,7 @@ from .registry import (
     register_norm, register_position_encoding, register_stream_op,
 )
 from .context import BiasedDelta, BuildEnv, LayerCache, ResidualStream, StepContext
-from . import norm, rope, attention, swiglu, dense, block, embedding, gate, stream_ops, gla, moe  # noqa: F401  (registers the built-in kinds)
+from . import norm, rope, attention, swiglu, dense, block, embedding, gate, stream_ops, gla, moe, ssm, hgrn, latent_attention  # noqa: F401  (registers the built-in kinds)
 from .model import DecoderModel
 
 __all__ = [

@@ -101,3 +101,29 @@ class GatedPreNormBlock:
             logits = self.feed_forward_gate.logits(h)
             stream.delta = self.feed_forward.forward(h, ctx)
             stream.gate = (logits, self.feed_forward_gate.bias)
+
+
+@register_block("sandwich")
+class SandwichBlock:
+    """``x += post1(mixer(norm1(x)))``, then ``x += post2(feed_forward(norm2(x)))`` if the layer has a feed-forward:
+    a norm in front of each sublayer and another on its result.  The result travels as the stream's pending delta
+    with its norm (``stream.post``); the norm in front of the next sublayer (or the model's last) norms it, adds it
+    into the float32 residual and norms the sum for its own sublayer, in one kernel where both norms are of a kind
+    whose kernel can (``dyt``)."""
+
+    def __init__(self, mixer, mixer_norm, mixer_post_norm, feed_forward=None, feed_forward_norm=None,
+                 feed_forward_post_norm=None):
+        if not ((feed_forward is None) == (feed_forward_norm is None) == (feed_forward_post_norm is None)):
+            raise ValueError("a sandwich block has a feed-forward with both of its norms, or none of them")
+        self.mixer, self.mixer_norm, self.mixer_post_norm = mixer, mixer_norm, mixer_post_norm
+        self.feed_forward, self.feed_forward_norm = feed_forward, feed_forward_norm
+        self.feed_forward_post_norm = feed_forward_post_norm
+
+    def forward(self, stream, ctx, cache):
+        h = self.mixer_norm.forward(stream)
+        stream.delta = self.mixer.forward(h, ctx, cache)
+        stream.post = self.mixer_post_norm
+        if self.feed_forward is not None:
+            h = self.feed_forward_norm.forward(stream)
+            stream.delta = self.feed_forward.forward(h, ctx)
+            stream.post = self.feed_forward_post_norm

@@ -79,15 +79,21 @@ class ResidualStream:
     on its way into the residual (``residual += delta * sigmoid(logits + bias)``).  It is set after the delta and
     forgotten with it; whoever adds the delta (a norm, ``settle``) reads it.  A delta may also be a
     ``BiasedDelta``: a result whose bias is still to be added, which the gated add takes in passing.
+
+    ``post`` belongs to the pending delta too: a norm part that the delta passes on its way into the residual
+    (``residual += post(delta)``, for blocks that norm a sublayer's result as well as its input).  It is set after
+    the delta and forgotten with it; a norm that can apply it inside its own kernel does so, everybody else has it
+    applied by ``settle`` (the norm's ``add_normed``).
     """
 
-    __slots__ = ("residual", "raw_delta", "lowered", "gate")
+    __slots__ = ("residual", "raw_delta", "lowered", "gate", "post")
 
     def __init__(self, residual: torch.Tensor, delta: Optional[torch.Tensor] = None):
         self.residual = residual
         self.raw_delta = delta
         self.lowered = None
         self.gate = None
+        self.post = None
 
     @property
     def delta(self):
@@ -99,6 +105,7 @@ class ResidualStream:
     def delta(self, value):
         self.raw_delta = value
         self.gate = None
+        self.post = None
         if value is not None:
             self.lowered = None
 
@@ -106,6 +113,11 @@ class ResidualStream:
         """Adds what is pending into the residual (no norm follows) and returns the residual."""
         raw = self.raw_delta
         if raw is None:
+            return self.residual
+        if self.post is not None:
+            post = self.post
+            post.add_normed(self, raw)
+            self.delta = None
             return self.residual
         bias = None
         if isinstance(raw, BiasedDelta):

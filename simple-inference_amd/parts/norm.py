@@ -58,6 +58,8 @@ class RMSNorm:
         product's own kernel, and the product after the norm divides: the norm has no kernel of its own.
         """
         k = self.env.kernels
+        if stream.post is not None:     # the pending result passes a norm of its own first: that norm's kernel adds it
+            stream.settle(k)
         if stream.gate is not None or isinstance(stream.raw_delta, BiasedDelta):
             return self._gated(stream, rows)
         if scaled_ok and rows is None and hasattr(stream.raw_delta, "compute") and hasattr(k, "linear_into_residual"):
@@ -85,6 +87,64 @@ class RMSNorm:
         else:
             out = self.env.kernels.add_rmsnorm(stream.residual, raw, self.weight, self.eps, self.env.dtype, rows,
                                                gate=logits, gate_bias=gate_bias, delta_bias=bias)
+        if rows is None:
+            stream.delta = None
+        return out
+
+
+@register_norm("dyt")
+class DynamicTanh:
+    """A norm without a statistic: ``y = tanh(a * x) * w + b`` with a learned scalar ``a``, elementwise, in float32
+    with one rounding.  With ``scaled`` it has a second vector ``s`` and gives ``(tanh(a * x) * w + b) * s`` (a layer
+    scale on a sublayer's normed result).
+
+    params: size, and optionally scaled (default False).
+
+    In front of a sublayer (``forward``) it first adds what is pending into the float32 residual; a pending result
+    that passes a norm of this kind on its way (``stream.post``) is normed and added in the same kernel.  Behind a
+    sublayer (``add_normed``) it adds its own output into the residual.
+    """
+
+    def __init__(self, params, env):
+        self.size = int(params["size"])
+        self.scaled = bool(params.get("scaled", False))
+        self.env = env
+        self.weight = self.bias = self.alpha = self.scale = None
+
+    def weight_specs(self):
+        specs = {"weight": TensorSpec((self.size,), "vector"), "bias": TensorSpec((self.size,), "vector"),
+                 "alpha": TensorSpec((), "vector")}
+        if self.scaled:
+            specs["scale"] = TensorSpec((self.size,), "vector")
+        return specs
+
+    def bind(self, tensors):
+        self.weight, self.bias = tensors["weight"].contiguous(), tensors["bias"].contiguous()
+        self.alpha = tensors["alpha"].reshape(1).contiguous()
+        self.scale = tensors["scale"].contiguous() if self.scaled else None
+
+    def terms(self):
+        """(weight, bias, alpha, scale or None): what the kernels need of this norm."""
+        return (self.weight, self.bias, self.alpha, self.scale)
+
+    def add_normed(self, stream, y):
+        """``stream.residual += norm(y)``; returns nothing (no sublayer reads the un-normed residual)."""
+        if hasattr(y, "compute"):
+            y = y.compute()
+        self.env.kernels.dyt_norm(stream.residual, y, self.terms(), None, self.env.dtype)
+
+    def forward(self, stream, rows=None, scaled_ok=False):
+        """Adds what is pending into ``stream.residual`` and returns the normed rows; with ``rows`` (int32 indices)
+        only those rows are computed and the residual is left as it was."""
+        k = self.env.kernels
+        post = stream.post
+        if stream.gate is not None or isinstance(stream.raw_delta, BiasedDelta) or (
+                post is not None and not isinstance(post, DynamicTanh)):
+            stream.settle(k)
+            post = None
+        delta = stream.delta
+        out = k.dyt_norm(stream.residual, delta, post.terms() if (post is not None and delta is not None) else None,
+                         self.terms(), self.env.dtype, rows)
         if rows is None:
             stream.delta = None
         return out

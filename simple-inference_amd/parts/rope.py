@@ -9,6 +9,10 @@ floats on the float32 values, as the reference's does.  Angles are
 ``float32(position) * inv_freq`` and the cos/sin tables stay float32.  The
 rotation itself pairs element ``i`` with ``i + d/2`` (reference:
 ``ops/rope.py:167-182``) and is applied by the kernel that also writes the cache.
+
+Two further forms, each a parameter: ``scaling["rope_type"] == "yarn"`` stretches the frequencies by a ramp over the
+pair index and raises the amplitude of both tables (see ``yarn_inv_freq``); ``pairing == "interleaved"`` says that a
+consumer pairs element ``2i`` with ``2i + 1`` (the tables are the same; the kernel that rotates reads the flag).
 """
 
 from __future__ import annotations
@@ -44,9 +48,28 @@ def rotary_inv_freq(rotary_dim: int, theta: float, scaling=None) -> torch.Tensor
     return torch.tensor(scaled, dtype=torch.float32)
 
 
+def yarn_inv_freq(rotary_dim: int, theta: float, scaling) -> tuple:
+    """Frequencies and table amplitude of the ramp form.  With ``turn(t) = d * ln(original / (2 pi t)) / (2 ln theta)``
+    (the pair index whose wave makes ``t`` turns over ``original`` positions), ``lo = max(floor(turn(fast)), 0)``,
+    ``hi = min(ceil(turn(slow)), d - 1)`` and ``ramp_i = clamp((i - lo) / max(hi - lo, 0.001), 0, 1)``, pair ``i``
+    turns at ``f_i / factor * ramp_i + f_i * (1 - ramp_i)``; cos and sin are multiplied by ``0.1 ln(factor) + 1``."""
+    idx = torch.arange(0, rotary_dim, 2, dtype=torch.float64)
+    f = theta ** (-idx / rotary_dim)
+    factor, original = float(scaling["factor"]), float(scaling["original"])
+
+    def turn(t):
+        return rotary_dim * math.log(original / (2 * math.pi * t)) / (2 * math.log(theta))
+
+    lo = max(math.floor(turn(float(scaling["fast"]))), 0)
+    hi = min(math.ceil(turn(float(scaling["slow"]))), rotary_dim - 1)
+    ramp = ((torch.arange(rotary_dim // 2, dtype=torch.float64) - lo) / max(hi - lo, 0.001)).clamp(0, 1)
+    return f / factor * ramp + f * (1 - ramp), 0.1 * math.log(factor) + 1.0
+
+
 @register_position_encoding("rope")
 class RotaryEncoding:
-    """params: rotary_dim, theta, scaling (dict or None)."""
+    """params: rotary_dim, theta, scaling (dict or None), and optionally pairing ("half", the default, or
+    "interleaved")."""
 
     def __init__(self, params, env):
         self.rotary_dim = int(params["rotary_dim"])
@@ -54,6 +77,9 @@ class RotaryEncoding:
             raise ValueError(f"rotary_dim must be even, got {self.rotary_dim}")
         self.theta = float(params["theta"])
         self.scaling = params.get("scaling")
+        self.pairing = str(params.get("pairing", "half"))
+        if self.pairing not in ("half", "interleaved"):
+            raise ValueError(f"pairing must be 'half' or 'interleaved', got {self.pairing!r}")
         self.max_positions = int(env.max_positions)
         self.device = env.device
         self._tables = None
@@ -67,11 +93,19 @@ class RotaryEncoding:
     def tables(self):
         """(cos, sin), each float32 ``[max_positions, rotary_dim/2]``, on the device."""
         if self._tables is None:
-            inv_freq = rotary_inv_freq(self.rotary_dim, self.theta, self.scaling)
-            pos = torch.arange(self.max_positions, dtype=torch.float32)
+            amplitude = 1.0
+            if self.scaling is not None and self.scaling.get("rope_type") == "yarn":
+                inv_freq, amplitude = yarn_inv_freq(self.rotary_dim, self.theta, self.scaling)
+            else:
+                inv_freq = rotary_inv_freq(self.rotary_dim, self.theta, self.scaling)
+            # the ramp form's angles are taken in float64 on the host and the tables rounded once
+            pos = torch.arange(self.max_positions, dtype=inv_freq.dtype)
             angles = torch.outer(pos, inv_freq)
-            self._tables = (angles.cos().to(self.device).contiguous(),
-                            angles.sin().to(self.device).contiguous())
+            cos, sin = angles.cos(), angles.sin()
+            if amplitude != 1.0:
+                cos, sin = cos * amplitude, sin * amplitude
+            cos, sin = cos.float(), sin.float()
+            self._tables = (cos.to(self.device).contiguous(), sin.to(self.device).contiguous())
         return self._tables
 
 

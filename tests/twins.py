@@ -109,9 +109,151 @@ class TwinKernels:
         out = out * torch.rsqrt(out.pow(2).mean(-1, keepdim=True) + eps) * norm_weight.float()
         return (out.view(N, H * Dv) * torch.nn.functional.silu(g)).to(proj.dtype)
 
+    # -- norm without a statistic ------------------------------------------------------
+    @staticmethod
+    def _dyt(x, terms):
+        w, b, alpha, scale = terms
+        y = torch.tanh(alpha.float() * x.float()) * w.float() + b.float()
+        return y * scale.float() if scale is not None else y
+
+    def dyt_norm(self, residual, delta, post, pre, out_dtype, rows=None):
+        add = None
+        if delta is not None:
+            add = self._dyt(delta, post) if post is not None else delta.float()
+        if rows is None:
+            if add is not None:
+                residual.add_(add)
+            x = residual
+        else:
+            x = residual[rows.long()]
+            if add is not None:
+                x = x + add[rows.long()]
+        return self._dyt(x, pre).to(out_dtype) if pre is not None else None
+
+    # -- short convolution and recurrences with a state -------------------------------------
+    def causal_conv(self, proj, first_col, weight, bias, activation, ctx, state, state_offset):
+        channels, taps = weight.shape
+        u = proj[:, first_col:first_col + channels].float()
+        out = torch.zeros_like(u)
+        cu, slots = ctx.cu_q.tolist(), ctx.state_slots.tolist()
+        w = weight.float()
+        for s in range(ctx.n_seqs):
+            past = state[slots[s], state_offset:state_offset + channels * (taps - 1)].view(taps - 1, channels)
+            seq = torch.cat([past, u[cu[s]:cu[s + 1]]], dim=0)
+            n = cu[s + 1] - cu[s]
+            acc = bias.float().expand(n, channels).clone()
+            for j in range(taps):
+                acc += seq[j:j + n] * w[:, j]
+            out[cu[s]:cu[s + 1]] = acc
+            if taps > 1:
+                past.copy_(seq[n:])
+        if activation == "silu":
+            out = torch.nn.functional.silu(out)
+        return out.to(proj.dtype)
+
+    def ssd_scan(self, proj, xbc, dt_bias, a_log, d_skip, norm_weight, n_heads, head_dim, state_size, groups,
+                 norm_groups, eps, ctx, state):
+        n, H, P, N, G = proj.shape[0], n_heads, head_dim, state_size, groups
+        inner = H * P
+        z = proj[:, :inner].float()
+        dt = torch.nn.functional.softplus(proj[:, proj.shape[1] - H:].float() + dt_bias.float(), threshold=1e9)
+        decay = torch.exp(-torch.exp(a_log.float()) * dt)
+        x = xbc[:, :inner].float().view(n, H, P)
+        B = xbc[:, inner:inner + G * N].float().view(n, G, N).repeat_interleave(H // G, dim=1)
+        C = xbc[:, inner + G * N:].float().view(n, G, N).repeat_interleave(H // G, dim=1)
+        y = torch.zeros(n, H, P)
+        cu, slots = ctx.cu_q.tolist(), ctx.state_slots.tolist()
+        for s in range(ctx.n_seqs):
+            S = state[slots[s], :H * N * P].view(H, N, P)
+            for t in range(cu[s], cu[s + 1]):
+                S.mul_(decay[t][:, None, None]).add_((dt[t][:, None] * B[t])[:, :, None] * x[t][:, None, :])
+                y[t] = torch.einsum("hn,hnp->hp", C[t], S)
+        y = (y + d_skip.float()[None, :, None] * x).view(n, inner) * torch.nn.functional.silu(z)
+        parts = y.view(n, norm_groups, inner // norm_groups)
+        y = (parts * torch.rsqrt(parts.pow(2).mean(-1, keepdim=True) + eps)).view(n, inner) * norm_weight.float()
+        return y.to(proj.dtype)
+
+    def hgrn2_scan(self, proj, f_bias, lower, norm_weight, n_heads, key_dim, value_dim, eps, ctx, state):
+        n, H, D, Dv = proj.shape[0], n_heads, key_dim, value_dim
+        p = proj.float()
+        q = torch.nn.functional.silu(p[:, :H * D]).to(proj.dtype).float().view(n, H, D)
+        low = lower.float()
+        f = (low + (1 - low) * torch.sigmoid(p[:, H * D:2 * H * D] + f_bias.float())).view(n, H, D)
+        v = p[:, 2 * H * D:].view(n, H, Dv)
+        out = torch.zeros(n, H, Dv)
+        cu, slots = ctx.cu_q.tolist(), ctx.state_slots.tolist()
+        for s in range(ctx.n_seqs):
+            S = state[slots[s]]
+            for t in range(cu[s], cu[s + 1]):
+                S.mul_(f[t][:, :, None]).add_((1 - f[t])[:, :, None] * v[t][:, None, :])
+                out[t] = torch.einsum("hd,hdv->hv", q[t], S)
+        out = out * torch.rsqrt(out.pow(2).mean(-1, keepdim=True) + eps) * norm_weight.float()
+        return out.view(n, H * Dv).to(proj.dtype)
+
+    # -- latent attention ------------------------------------------------------------------
+    @staticmethod
+    def _rotate_pairs(x, rotary_dim, cos, sin, pos):
+        """``x [n, ..., r]`` float: neighbouring pairs of the first ``rotary_dim`` elements turned by the tables' rows."""
+        if rotary_dim == 0:
+            return x
+        shape = [x.shape[0]] + [1] * (x.dim() - 2) + [rotary_dim // 2]
+        c, s = cos[pos.long()].view(shape), sin[pos.long()].view(shape)
+        a, b = x[..., 0:rotary_dim:2], x[..., 1:rotary_dim:2]
+        out = x.clone()
+        out[..., 0:rotary_dim:2] = a * c - b * s
+        out[..., 1:rotary_dim:2] = b * c + a * s
+        return out
+
+    def latent_prepare(self, proj, q_rank, q_gain, kv_rank, kv_gain, rot_dim, rotary_dim, cos, sin, eps, ctx, cache,
+                       page_dim=None):
+        p = proj.float()
+        cq = p[:, :q_rank]
+        cq = (cq * torch.rsqrt(cq.pow(2).mean(-1, keepdim=True) + eps) * q_gain.float()).to(proj.dtype)
+        if kv_rank:
+            a = p[:, q_rank:q_rank + kv_rank]
+            c = (a * torch.rsqrt(a.pow(2).mean(-1, keepdim=True) + eps) * kv_gain.float()).to(proj.dtype)
+            b = self._rotate_pairs(p[:, q_rank + kv_rank:q_rank + kv_rank + rot_dim], rotary_dim, cos, sin,
+                                   ctx.positions).to(proj.dtype)
+            pos = ctx.positions.long()
+            ps = cache.page_size
+            page = cache.block_table.long()[ctx.seq_of_token.long(), pos // ps]
+            off = pos % ps
+            cache.k_pages[page, 0, off, :kv_rank] = c
+            cache.k_pages[page, 0, off, kv_rank:kv_rank + rot_dim] = b
+            cache.v_pages[page, 0, :kv_rank, off] = c
+        return cq
+
+    def headwise_linear(self, x, w, in_stride, out_stride, tail=0, rotation=None):
+        n = x.shape[0]
+        H, out_dim, in_dim = w.shape
+        xs = x.float().view(n, H, in_stride)
+        y = torch.zeros(n, H, out_stride)
+        y[:, :, :out_dim] = torch.einsum("nhi,hoi->nho", xs[:, :, :in_dim], w.float())
+        if tail:
+            t = xs[:, :, in_dim:in_dim + tail]
+            if rotation is not None:
+                rotary_dim, cos, sin, positions = rotation
+                t = self._rotate_pairs(t, rotary_dim, cos, sin, positions)
+            y[:, :, out_dim:out_dim + tail] = t
+        return y.view(n, H * out_stride).to(x.dtype)
+
     # -- mixture of experts ---------------------------------------------------------
-    def moe_route(self, h, router, top):
+    def moe_route(self, h, router, top, score="softmax", groups=None, scale=1.0):
         logits = h.float() @ router.float().T
+        if score == "sigmoid":
+            sc = torch.sigmoid(logits)
+            ranked = sc
+            if groups is not None:
+                count, keep = groups
+                per = sc.shape[1] // count
+                g = sc.view(-1, count, per)
+                gscore = torch.sort(g, dim=-1, descending=True).values[:, :, :2].sum(-1)
+                best = torch.sort(gscore, dim=-1, descending=True, stable=True).indices[:, :keep]
+                allowed = torch.zeros_like(gscore, dtype=torch.bool).scatter_(1, best, True)
+                ranked = sc.masked_fill(~allowed[:, :, None].expand(-1, -1, per).reshape(sc.shape), -1.0)
+            order = torch.sort(ranked, dim=-1, descending=True, stable=True).indices[:, :top]
+            chosen = torch.gather(sc, 1, order)
+            return order.to(torch.int32), chosen / (chosen.sum(-1, keepdim=True) + 1e-20) * scale
         order = torch.sort(logits, dim=-1, descending=True, stable=True).indices[:, :top]
         best = torch.gather(logits, 1, order)
         return order.to(torch.int32), torch.softmax(best, -1)
