@@ -1,7 +1,8 @@
 // Mixture of experts: the router, and the experts' products for a token's chosen experts.
 //
 //   route:    z = R h (float, R float [E, width]); the ``top`` largest logits (ties: the lower index) and the softmax
-//             over those alone:  ids [N, top] int32,  weights [N, top] float
+//             over those alone:  ids [N, top] int32,  weights [N, top] float; or sigmoid scores, the choice among the
+//             best groups of experts, weights normalised over the chosen and scaled
 //   gate/up:  a[s, f] = silu(h[n] . Wg[e][f]) * (h[n] . Wu[e][f])      s = n * top + k, e = ids[s]
 //             the experts' matrices are stacked: W1 [E, 2 * ff, width], gate rows first
 //   down:     y[n, c] = sum_k weights[n, k] * (a[n * top + k] . W2[e_k][c])  (+ sigmoid(sg[n]) * shared[n, c])
@@ -14,11 +15,17 @@
 #define MOE_MAX_EXPERTS 1024
 #define MOE_MAX_TOP 64
 
+// score_mode 0: the softmax over the chosen logits alone.  score_mode 1: scores s = sigmoid(z); with n_groups > 0 the
+// experts form n_groups equal groups of neighbours, a group's score is the sum of its two largest s, and only
+// experts of the keep_groups best groups (ties: the lower group) can be chosen; the weights are the chosen s divided
+// by their sum (+ 1e-20), times weight_scale.
 template <typename T>
 __global__ __launch_bounds__(256) void moe_route_kernel(const T* __restrict__ h, const float* __restrict__ router,
                                                          int* __restrict__ ids, float* __restrict__ weights, int width,
-                                                         int n_experts, int top) {
+                                                         int n_experts, int top, int score_mode, int n_groups,
+                                                         int keep_groups, float weight_scale) {
     __shared__ float logit_s[MOE_MAX_EXPERTS];
+    __shared__ float group_s[MOE_MAX_EXPERTS];
     const int n = blockIdx.x, wave = threadIdx.x / SIA_WAVE, lane = threadIdx.x % SIA_WAVE;
     const T* x = h + (size_t)n * width;
     // a wave an expert at a time; four independent runs of loads a lane, so that a row's latency is paid once
@@ -32,10 +39,47 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const T* __restrict__ h,
         }
         for (; i < width; i += SIA_WAVE) acc[0] += to_float(x[i]) * w[i];
         const float total = wave_sum((acc[0] + acc[1]) + (acc[2] + acc[3]));
-        if (lane == 0) logit_s[e] = total;
+        if (lane == 0) logit_s[e] = score_mode == 1 ? 1.f / (1.f + expf(-total)) : total;
     }
     __syncthreads();
     if (wave != 0) return;
+    if (score_mode == 1 && n_groups > 0) {
+        // a lane a group at a time: the sum of its two largest scores; then keep_groups rounds of a wave-wide best
+        // group, and the experts of every other group leave the choice
+        const int per = n_experts / n_groups;
+        for (int g = lane; g < n_groups; g += SIA_WAVE) {
+            float a = -INFINITY, b = -INFINITY;
+            for (int e = g * per; e < (g + 1) * per; ++e) {
+                const float z = logit_s[e];
+                if (z > a) { b = a; a = z; } else if (z > b) { b = z; }
+            }
+            group_s[g] = per > 1 ? a + b : a;
+        }
+        __builtin_amdgcn_wave_barrier();
+        __threadfence_block();
+        for (int k = 0; k < keep_groups; ++k) {
+            float best = -INFINITY;
+            int which = 0x7fffffff;
+            for (int g = lane; g < n_groups; g += SIA_WAVE) {
+                const float z = group_s[g];
+                if (z > best) { best = z; which = g; }
+            }
+#pragma unroll
+            for (int off = SIA_WAVE / 2; off > 0; off >>= 1) {
+                const float ob = __shfl_xor(best, off, SIA_WAVE);
+                const int ow = __shfl_xor(which, off, SIA_WAVE);
+                if (ob > best || (ob == best && ow < which)) { best = ob; which = ow; }
+            }
+            if (which >= n_groups) break;
+            if (lane == 0) group_s[which] = INFINITY;      // kept
+            __builtin_amdgcn_wave_barrier();
+            __threadfence_block();
+        }
+        for (int e = lane; e < n_experts; e += SIA_WAVE)
+            if (group_s[e / per] != INFINITY) logit_s[e] = -INFINITY;
+        __builtin_amdgcn_wave_barrier();
+        __threadfence_block();
+    }
     float chosen = 0.f, first = 0.f, total = 0.f;   // lane k keeps the k-th choice
     int chosen_id = 0;
     for (int k = 0; k < top; ++k) {
@@ -51,9 +95,9 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const T* __restrict__ h,
             const int ow = __shfl_xor(which, off, SIA_WAVE);
             if (ob > best || (ob == best && ow < which)) { best = ob; which = ow; }
         }
-        if (which >= n_experts) which = k;   // logits that are not numbers order nothing: still an expert that exists
+        if (which >= n_experts) { which = k; best = 0.f; }   // logits that are not numbers order nothing: still an expert that exists
         if (k == 0) first = best;
-        const float p = expf(best - first);
+        const float p = score_mode == 1 ? best : expf(best - first);
         total += p;
         if (lane == k) { chosen = p; chosen_id = which; }
         if (lane == 0 && which < n_experts) logit_s[which] = -INFINITY;
@@ -62,25 +106,34 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const T* __restrict__ h,
     }
     if (lane < top) {
         ids[(size_t)n * top + lane] = chosen_id;
-        weights[(size_t)n * top + lane] = chosen / total;
+        weights[(size_t)n * top + lane] = score_mode == 1 ? chosen / (total + 1e-20f) * weight_scale : chosen / total;
     }
 }
 
-SIA_EXPORT int sia_moe_route(const void* h, const float* router, int* ids, float* weights, int n_tokens, int width,
-                             int n_experts, int top, int dtype, hipStream_t stream) {
+SIA_EXPORT int sia_moe_route_ex(const void* h, const float* router, int* ids, float* weights, int n_tokens, int width,
+                                int n_experts, int top, int dtype, int score_mode, int n_groups, int keep_groups,
+                                float weight_scale, hipStream_t stream) {
     if (n_tokens <= 0) return 0;
-    if (n_experts <= 0 || n_experts > MOE_MAX_EXPERTS || top <= 0 || top > n_experts || top > MOE_MAX_TOP)
+    if (n_experts <= 0 || n_experts > MOE_MAX_EXPERTS || top <= 0 || top > n_experts || top > MOE_MAX_TOP ||
+        (score_mode != 0 && score_mode != 1) || n_groups < 0 ||
+        (n_groups > 0 && (score_mode != 1 || n_experts % n_groups || keep_groups <= 0 || keep_groups > n_groups ||
+                          top > n_experts / n_groups * keep_groups)))
         return SIA_BAD_ARGUMENT;
     dim3 grid(n_tokens), block(256);
     if (dtype == SIA_F32)
         hipLaunchKernelGGL(moe_route_kernel<float>, grid, block, 0, stream, (const float*)h, router, ids, weights, width,
-                           n_experts, top);
+                           n_experts, top, score_mode, n_groups, keep_groups, weight_scale);
     else if (dtype == SIA_BF16)
         hipLaunchKernelGGL(moe_route_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)h, router, ids, weights,
-                           width, n_experts, top);
+                           width, n_experts, top, score_mode, n_groups, keep_groups, weight_scale);
     else
         return SIA_BAD_ARGUMENT;
     return SIA_LAUNCH_CHECK();
+}
+
+SIA_EXPORT int sia_moe_route(const void* h, const float* router, int* ids, float* weights, int n_tokens, int width,
+                             int n_experts, int top, int dtype, hipStream_t stream) {
+    return sia_moe_route_ex(h, router, ids, weights, n_tokens, width, n_experts, top, dtype, 0, 0, 0, 1.f, stream);
 }
 
 // dot product of two rows of K elements by one wave (every lane gets the sum)

@@ -33,7 +33,7 @@ __global__ __launch_bounds__(512) void gla_recurrent_kernel(
     const T* __restrict__ proj, int row_stride, int q_col, int k_col, int v_col, int g_col,
     const float* __restrict__ alpha, const float* __restrict__ norm_w, float* __restrict__ state, const int* __restrict__ cu_q, const int* __restrict__ slots, T* __restrict__ out,
     int n_heads, int D, int Dv, int R, int block_tokens, float q_scale, float eps, int slice,
-    float* __restrict__ raw_out) {
+    float* __restrict__ raw_out, const float* __restrict__ k_f32, int q_share, long long state_stride) {
     extern __shared__ float lds[];
     const int seq = blockIdx.x, head = blockIdx.y, tid = threadIdx.x;
     const int j0 = blockIdx.z * slice;     // this workgroup's columns: j0 .. j0 + slice - 1
@@ -49,7 +49,7 @@ __global__ __launch_bounds__(512) void gla_recurrent_kernel(
 
     const int j = j0 + tid / R, r = tid % R;
     const bool owns = tid / R < slice && j < Dv;
-    float* S_mem = state + ((size_t)slots[seq] * n_heads + head) * D * Dv;
+    float* S_mem = state + (size_t)slots[seq] * state_stride + (size_t)head * D * Dv;
     float S[ROWS];
 #pragma unroll
     for (int i = 0; i < ROWS; ++i) {
@@ -57,6 +57,7 @@ __global__ __launch_bounds__(512) void gla_recurrent_kernel(
         S[i] = (owns && d < D) ? S_mem[(size_t)d * Dv + j] : 0.f;
     }
     const int wave = tid / SIA_WAVE, lane = tid % SIA_WAVE, n_waves = blockDim.x / SIA_WAVE;
+    const int q_head = head / q_share;      // q (and a k read from the rows) may be shared by q_share neighbouring heads
 
     for (int t0 = first; t0 < last; t0 += TB) {
         const int nt = min(TB, last - t0);
@@ -64,13 +65,14 @@ __global__ __launch_bounds__(512) void gla_recurrent_kernel(
             const int t = idx / Dv, c = idx % Dv;
             const T* row = proj + (size_t)(t0 + t) * row_stride;
             v_s[t * Dv + c] = to_float(row[v_col + head * Dv + c]);
-            g_s[t * Dv + c] = to_float(row[g_col + head * Dv + c]);
+            g_s[t * Dv + c] = g_col >= 0 ? to_float(row[g_col + head * Dv + c]) : 0.f;
         }
         for (int idx = tid; idx < nt * D; idx += blockDim.x) {
             const int t = idx / D, c = idx % D;
             const T* row = proj + (size_t)(t0 + t) * row_stride;
-            q_s[t * D + c] = to_float(row[q_col + head * D + c]) * q_scale;
-            k_s[t * D + c] = to_float(row[k_col + head * D + c]);
+            q_s[t * D + c] = to_float(row[q_col + q_head * D + c]) * q_scale;
+            k_s[t * D + c] = k_f32 ? k_f32[((size_t)(t0 + t) * n_heads + head) * D + c]
+                                   : to_float(row[k_col + q_head * D + c]);
             al_s[t * D + c] = alpha[((size_t)(t0 + t) * n_heads + head) * D + c];
         }
         __syncthreads();
@@ -100,7 +102,7 @@ __global__ __launch_bounds__(512) void gla_recurrent_kernel(
             T* dst = out + ((size_t)(t0 + t) * n_heads + head) * Dv;
             for (int c = lane; c < Dv; c += SIA_WAVE) {
                 const float g = g_s[t * Dv + c];
-                dst[c] = from_float<T>(o_s[t * Dv + c] * inv * norm_w[c] * (g / (1.f + expf(-g))));
+                dst[c] = from_float<T>(o_s[t * Dv + c] * inv * norm_w[c] * (g_col >= 0 ? g / (1.f + expf(-g)) : 1.f));
             }
         }
         __syncthreads();
@@ -347,11 +349,11 @@ __global__ __launch_bounds__(SIA_WAVE) void gla_finish_kernel(const float* __res
     float ss = 0.f;
     for (int c = lane; c < Dv; c += SIA_WAVE) ss += o[c] * o[c];
     const float inv = rsqrtf(wave_sum(ss) / (float)Dv + eps);
-    const T* g_row = proj + (size_t)n * row_stride + g_col + head * Dv;
+    const T* g_row = proj + (size_t)n * row_stride + (g_col >= 0 ? g_col : 0) + head * Dv;
     T* dst = out + ((size_t)n * n_heads + head) * Dv;
     for (int c = lane; c < Dv; c += SIA_WAVE) {
-        const float g = to_float(g_row[c]);
-        dst[c] = from_float<T>(o[c] * inv * norm_w[c] * (g / (1.f + expf(-g))));
+        const float g = g_col >= 0 ? to_float(g_row[c]) : 0.f;
+        dst[c] = from_float<T>(o[c] * inv * norm_w[c] * (g_col >= 0 ? g / (1.f + expf(-g)) : 1.f));
     }
 }
 
@@ -370,30 +372,18 @@ SIA_EXPORT long long sia_gla_workspace(int n_tokens, int n_seqs, int max_q_len, 
     return (long long)n_tokens * n_heads * D + (long long)n_tokens * n_heads * Dv;
 }
 
-SIA_EXPORT int sia_gla_recurrent(const void* proj, int row_stride, int q_col, int k_col, int v_col, int g_col, int a_col,
-                                 const void* a2, const float* a2_bias, const float* norm_w, float* state,
-                                 const int* cu_q, const int* slots, void* out, int n_seqs, int max_q_len, int n_heads,
-                                 int D, int Dv, int rank, float tau, float q_scale, float eps, int dtype,
-                                 float* workspace, int n_tokens, hipStream_t stream) {
-    if (n_seqs <= 0) return 0;
-    if (D <= 0 || Dv <= 0 || D > 512 || Dv > 512 || rank <= 0 || rank > 1024 || n_heads <= 0 || n_heads > 65535 ||
-        !(tau > 0.f) || !state || !norm_w || !workspace || n_tokens <= 0)
-        return SIA_BAD_ARGUMENT;
-    float* alpha = workspace;
-    float* raw_space = workspace + (size_t)n_tokens * n_heads * D;
-    {
-        const int channels = n_heads * D;
-        dim3 dgrid((n_tokens + GLA_DECAY_TOKENS - 1) / GLA_DECAY_TOKENS, (channels + 255) / 256), dblock(256);
-        const size_t lds = (size_t)GLA_DECAY_TOKENS * rank * sizeof(float);
-        if (dtype == SIA_F32)
-            hipLaunchKernelGGL(gla_decay_kernel<float>, dgrid, dblock, lds, stream, (const float*)proj, row_stride, a_col,
-                               (const float*)a2, a2_bias, alpha, n_tokens, channels, rank, 1.f / tau);
-        else if (dtype == SIA_BF16)
-            hipLaunchKernelGGL(gla_decay_kernel<bf16_t>, dgrid, dblock, lds, stream, (const bf16_t*)proj, row_stride,
-                               a_col, (const bf16_t*)a2, a2_bias, alpha, n_tokens, channels, rank, 1.f / tau);
-        else
-            return SIA_BAD_ARGUMENT;
-    }
+// The recurrence itself for a step's runs of tokens, whoever prepared its inputs: S <- diag(alpha) S + k v^T, o = S^T q.
+// q and v (and k, unless k_f32 gives it as floats [tokens, heads, D]) are columns of rows of the compute type; head h
+// reads the q (and such a k) of head h / q_share.  A sequence's matrices lie state_stride floats apart from the next
+// slot's.  The outputs go to ``raw`` [tokens, heads, Dv] as floats if the caller wants them there (want_raw) or if a
+// head's columns are shared out between workgroups; otherwise they are normed over the head (norm_w, eps), gated by
+// silu of the columns at g_col (none if negative) and written to ``out``.  Returns through ``raw_used`` whether ``raw``
+// holds the outputs.
+static int launch_recurrence(const void* proj, int row_stride, int q_col, int k_col, int v_col, int g_col,
+                             const float* k_f32, int q_share, const float* alpha, const float* norm_w, float* state,
+                             long long state_stride, const int* cu_q, const int* slots, void* out, int n_seqs,
+                             int max_q_len, int n_heads, int D, int Dv, float q_scale, float eps, int dtype,
+                             float* raw_space, bool want_raw, bool* raw_used, hipStream_t stream) {
     // columns a workgroup: all of a head's, or with a workspace a slice of them, as narrow as it takes to fill the chip
     int slice = Dv;
     const bool prompt = gla_slices(n_seqs, max_q_len, n_heads);
@@ -425,10 +415,12 @@ SIA_EXPORT int sia_gla_recurrent(const void* proj, int row_stride, int q_col, in
     const int w_rows = (D + 15) / 16;
     const int w_rows_t = w_rows <= 4 ? 4 : w_rows <= 8 ? 8 : w_rows <= 16 ? 16 : 32;
     const size_t w_lds = (size_t)GLA_WALK_TOKENS * (3 * 16 * w_rows_t + 2 * w_slice) * sizeof(float);
-    const bool ahead = prompt && dtype == SIA_BF16 && D % 8 == 0 && row_stride % 8 == 0 && q_col % 8 == 0 &&
-                       k_col % 8 == 0 && ((uintptr_t)proj % 16) == 0 &&
+    const bool ahead = prompt && dtype == SIA_BF16 && !k_f32 && q_share == 1 &&
+                       state_stride == (long long)n_heads * D * Dv && D % 8 == 0 && row_stride % 8 == 0 &&
+                       q_col % 8 == 0 && k_col % 8 == 0 && ((uintptr_t)proj % 16) == 0 &&
                        GLA_WALK_TOKENS * (D / 8) <= 4 * GLA_WALK_THREADS && w_lds <= 60 * 1024 && w_rows_t <= 16;
-    float* raw = (sliced || ahead) ? raw_space : nullptr;
+    float* raw = (sliced || ahead || want_raw) ? raw_space : nullptr;
+    if (raw_used) *raw_used = raw != nullptr;
     if (ahead) {
         dim3 wgrid(n_seqs, n_heads, (Dv + w_slice - 1) / w_slice), wblock(GLA_WALK_THREADS);
 #define WALK(ROWS, COLS)                                                                                             \
@@ -442,7 +434,7 @@ SIA_EXPORT int sia_gla_recurrent(const void* proj, int row_stride, int q_col, in
 #define LAUNCH(T, ROWS)                                                                                              \
     hipLaunchKernelGGL((gla_recurrent_kernel<T, ROWS>), grid, block, bytes(TB), stream, (const T*)proj, row_stride,  \
                        q_col, k_col, v_col, g_col, alpha, norm_w, state, cu_q, slots, (T*)out, n_heads, D, Dv, R, TB,   \
-                       q_scale, eps, slice, raw)
+                       q_scale, eps, slice, raw, k_f32, q_share, state_stride)
 #define PICK(T)                                                                                                      \
     do {                                                                                                             \
         if (rows <= 4) LAUNCH(T, 4);                                                                                 \
@@ -458,14 +450,200 @@ SIA_EXPORT int sia_gla_recurrent(const void* proj, int row_stride, int q_col, in
 #undef PICK
 #undef LAUNCH
     }
+    return 0;
+}
+
+SIA_EXPORT int sia_gla_recurrent(const void* proj, int row_stride, int q_col, int k_col, int v_col, int g_col, int a_col,
+                                 const void* a2, const float* a2_bias, const float* norm_w, float* state,
+                                 const int* cu_q, const int* slots, void* out, int n_seqs, int max_q_len, int n_heads,
+                                 int D, int Dv, int rank, float tau, float q_scale, float eps, int dtype,
+                                 float* workspace, int n_tokens, hipStream_t stream) {
+    if (n_seqs <= 0) return 0;
+    if (D <= 0 || Dv <= 0 || D > 512 || Dv > 512 || rank <= 0 || rank > 1024 || n_heads <= 0 || n_heads > 65535 ||
+        !(tau > 0.f) || !state || !norm_w || !workspace || n_tokens <= 0)
+        return SIA_BAD_ARGUMENT;
+    float* alpha = workspace;
+    float* raw_space = workspace + (size_t)n_tokens * n_heads * D;
+    {
+        const int channels = n_heads * D;
+        dim3 dgrid((n_tokens + GLA_DECAY_TOKENS - 1) / GLA_DECAY_TOKENS, (channels + 255) / 256), dblock(256);
+        const size_t lds = (size_t)GLA_DECAY_TOKENS * rank * sizeof(float);
+        if (dtype == SIA_F32)
+            hipLaunchKernelGGL(gla_decay_kernel<float>, dgrid, dblock, lds, stream, (const float*)proj, row_stride, a_col,
+                               (const float*)a2, a2_bias, alpha, n_tokens, channels, rank, 1.f / tau);
+        else if (dtype == SIA_BF16)
+            hipLaunchKernelGGL(gla_decay_kernel<bf16_t>, dgrid, dblock, lds, stream, (const bf16_t*)proj, row_stride,
+                               a_col, (const bf16_t*)a2, a2_bias, alpha, n_tokens, channels, rank, 1.f / tau);
+        else
+            return SIA_BAD_ARGUMENT;
+    }
+    bool raw = false;
+    const int code = launch_recurrence(proj, row_stride, q_col, k_col, v_col, g_col, nullptr, 1, alpha, norm_w, state,
+                                       (long long)n_heads * D * Dv, cu_q, slots, out, n_seqs, max_q_len, n_heads, D, Dv,
+                                       q_scale, eps, dtype, raw_space, false, &raw, stream);
+    if (code) return code;
     if (raw) {
         dim3 fgrid(n_tokens, n_heads), fblock(SIA_WAVE);
         if (dtype == SIA_F32)
-            hipLaunchKernelGGL(gla_finish_kernel<float>, fgrid, fblock, 0, stream, raw, (const float*)proj, row_stride,
-                               g_col, norm_w, (float*)out, n_heads, Dv, eps);
+            hipLaunchKernelGGL(gla_finish_kernel<float>, fgrid, fblock, 0, stream, raw_space, (const float*)proj,
+                               row_stride, g_col, norm_w, (float*)out, n_heads, Dv, eps);
         else
-            hipLaunchKernelGGL(gla_finish_kernel<bf16_t>, fgrid, fblock, 0, stream, raw, (const bf16_t*)proj, row_stride,
-                               g_col, norm_w, (bf16_t*)out, n_heads, Dv, eps);
+            hipLaunchKernelGGL(gla_finish_kernel<bf16_t>, fgrid, fblock, 0, stream, raw_space, (const bf16_t*)proj,
+                               row_stride, g_col, norm_w, (bf16_t*)out, n_heads, Dv, eps);
     }
+    return SIA_LAUNCH_CHECK();
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// The gated linear recurrence whose forget gate also decides what is written:
+//   f = l + (1 - l) * sigmoid(z_f + b),  S <- diag(f) S + (1 - f) v^T,  o = S^T silu(z_q),  y = o * rsqrt(mean(o^2) + eps) * w
+// Rows are [z_q (H * D) | z_f (H * D) | v (H * Dv)].  A first kernel leaves f and 1 - f in the float workspace and
+// silu(z_q) in the rows' own q columns; then the recurrence above, without an output gate.
+template <typename T>
+__global__ __launch_bounds__(256) void hgrn2_prepare_kernel(T* __restrict__ proj, int row_stride,
+                                                            const float* __restrict__ f_bias,
+                                                            const float* __restrict__ lower, float* __restrict__ alpha,
+                                                            float* __restrict__ k_f32, int channels) {
+    const int n = blockIdx.x, c = blockIdx.y * blockDim.x + threadIdx.x;
+    if (c >= channels) return;
+    T* row = proj + (size_t)n * row_stride;
+    const float zq = to_float(row[c]);
+    row[c] = from_float<T>(zq / (1.f + expf(-zq)));
+    const float z = to_float(row[channels + c]) + (f_bias ? f_bias[c] : 0.f);
+    const float l = lower ? lower[c] : 0.f;
+    const float f = l + (1.f - l) * (1.f / (1.f + expf(-z)));
+    alpha[(size_t)n * channels + c] = f;
+    k_f32[(size_t)n * channels + c] = 1.f - f;
+}
+
+// floats of workspace: the gates and their complements [tokens, heads, D] each, the raw outputs [tokens, heads, Dv]
+SIA_EXPORT long long sia_hgrn2_workspace(int n_tokens, int n_heads, int D, int Dv) {
+    return 2LL * n_tokens * n_heads * D + (long long)n_tokens * n_heads * Dv;
+}
+
+SIA_EXPORT int sia_hgrn2_scan(void* proj, int row_stride, const float* f_bias, const float* lower, const float* norm_w,
+                              float* state, const int* cu_q, const int* slots, void* out, int n_tokens, int n_seqs,
+                              int max_q_len, int n_heads, int D, int Dv, float eps, int dtype, float* workspace,
+                              hipStream_t stream) {
+    if (n_seqs <= 0 || n_tokens <= 0) return 0;
+    if (D <= 0 || Dv <= 0 || D > 512 || Dv > 512 || n_heads <= 0 || n_heads > 65535 || !state || !norm_w || !workspace ||
+        row_stride < n_heads * (2 * D + Dv))
+        return SIA_BAD_ARGUMENT;
+    const int channels = n_heads * D;
+    float* alpha = workspace;
+    float* kf = alpha + (size_t)n_tokens * channels;
+    float* raw_space = kf + (size_t)n_tokens * channels;
+    dim3 pgrid(n_tokens, (channels + 255) / 256), pblock(256);
+    if (dtype == SIA_F32)
+        hipLaunchKernelGGL(hgrn2_prepare_kernel<float>, pgrid, pblock, 0, stream, (float*)proj, row_stride, f_bias, lower,
+                           alpha, kf, channels);
+    else if (dtype == SIA_BF16)
+        hipLaunchKernelGGL(hgrn2_prepare_kernel<bf16_t>, pgrid, pblock, 0, stream, (bf16_t*)proj, row_stride, f_bias,
+                           lower, alpha, kf, channels);
+    else
+        return SIA_BAD_ARGUMENT;
+    bool raw = false;
+    const int code = launch_recurrence(proj, row_stride, 0, 0, 2 * channels, -1, kf, 1, alpha, norm_w, state,
+                                       (long long)n_heads * D * Dv, cu_q, slots, out, n_seqs, max_q_len, n_heads, D, Dv,
+                                       1.f, eps, dtype, raw_space, false, &raw, stream);
+    if (code) return code;
+    if (raw) {
+        dim3 fgrid(n_tokens, n_heads), fblock(SIA_WAVE);
+        if (dtype == SIA_F32)
+            hipLaunchKernelGGL(gla_finish_kernel<float>, fgrid, fblock, 0, stream, raw_space, (const float*)proj,
+                               row_stride, -1, norm_w, (float*)out, n_heads, Dv, eps);
+        else
+            hipLaunchKernelGGL(gla_finish_kernel<bf16_t>, fgrid, fblock, 0, stream, raw_space, (const bf16_t*)proj,
+                               row_stride, -1, norm_w, (bf16_t*)out, n_heads, Dv, eps);
+    }
+    return SIA_LAUNCH_CHECK();
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// The state-space recurrence with one decay per head:
+//   dt = softplus(z_dt + dt_bias),  S <- exp(-exp(A_log) dt) S + (dt B) x^T,  y = S^T C + D x        S [N, P] per head
+//   out = y * silu(z), divided by the root mean square of each of norm_groups equal parts of the row, times w
+// z and z_dt are columns of the projected rows ([z (H * P) | ... | z_dt (H)], the step sizes last); x, B, C are the
+// convolved rows [x (H * P) | B (G * N) | C (G * N)], head h reading the B and C of group h / (H / G).  A first kernel
+// leaves the decays and dt * B in the float workspace, the recurrence leaves y there, a last kernel adds D x, gates
+// and norms.
+template <typename T>
+__global__ __launch_bounds__(256) void ssd_prepare_kernel(const T* __restrict__ proj, int row_stride, int dt_col,
+                                                          const T* __restrict__ xbc, int xbc_stride, int b_col,
+                                                          const float* __restrict__ dt_bias,
+                                                          const float* __restrict__ a_log, float* __restrict__ alpha,
+                                                          float* __restrict__ k_f32, int n_heads, int N, int share) {
+    const int n = blockIdx.x, idx = blockIdx.y * blockDim.x + threadIdx.x;
+    if (idx >= n_heads * N) return;
+    const int h = idx / N, c = idx % N;
+    const float z = to_float(proj[(size_t)n * row_stride + dt_col + h]) + (dt_bias ? dt_bias[h] : 0.f);
+    const float dt = fmaxf(z, 0.f) + log1pf(expf(-fabsf(z)));
+    alpha[(size_t)n * n_heads * N + idx] = expf(-expf(a_log[h]) * dt);
+    k_f32[(size_t)n * n_heads * N + idx] = dt * to_float(xbc[(size_t)n * xbc_stride + b_col + (h / share) * N + c]);
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void ssd_finish_kernel(const float* __restrict__ raw, const T* __restrict__ proj,
+                                                         int row_stride, const T* __restrict__ xbc, int xbc_stride,
+                                                         const float* __restrict__ d_skip,
+                                                         const float* __restrict__ norm_w, T* __restrict__ out,
+                                                         int inner, int P, int part, float eps) {
+    __shared__ float scratch[16];
+    const int n = blockIdx.x, c0 = blockIdx.y * part;
+    const float* y = raw + (size_t)n * inner;
+    const T* z = proj + (size_t)n * row_stride;
+    const T* x = xbc + (size_t)n * xbc_stride;
+    float ss = 0.f;
+    for (int c = c0 + threadIdx.x; c < c0 + part; c += blockDim.x) {
+        const float g = to_float(z[c]);
+        const float v = (y[c] + (d_skip ? d_skip[c / P] : 0.f) * to_float(x[c])) * (g / (1.f + expf(-g)));
+        ss += v * v;
+    }
+    const float inv = rsqrtf(block_sum(ss, scratch) / (float)part + eps);
+    for (int c = c0 + threadIdx.x; c < c0 + part; c += blockDim.x) {
+        const float g = to_float(z[c]);
+        const float v = (y[c] + (d_skip ? d_skip[c / P] : 0.f) * to_float(x[c])) * (g / (1.f + expf(-g)));
+        out[(size_t)n * inner + c] = from_float<T>(v * inv * norm_w[c]);
+    }
+}
+
+SIA_EXPORT long long sia_ssd_workspace(int n_tokens, int n_heads, int N, int P) {
+    return 2LL * n_tokens * n_heads * N + (long long)n_tokens * n_heads * P;
+}
+
+SIA_EXPORT int sia_ssd_scan(const void* proj, int row_stride, const void* xbc, int xbc_stride, const float* dt_bias,
+                            const float* a_log, const float* d_skip, const float* norm_w, float* state,
+                            long long state_stride, const int* cu_q, const int* slots, void* out, int n_tokens,
+                            int n_seqs, int max_q_len, int n_heads, int P, int N, int groups, int norm_groups, float eps,
+                            int dtype, float* workspace, hipStream_t stream) {
+    if (n_seqs <= 0 || n_tokens <= 0) return 0;
+    const int inner = n_heads * P;
+    if (N <= 0 || P <= 0 || N > 512 || P > 512 || n_heads <= 0 || n_heads > 65535 || groups <= 0 || n_heads % groups ||
+        norm_groups <= 0 || inner % norm_groups || norm_groups > 65535 || !state || !norm_w || !a_log || !workspace ||
+        row_stride < inner + n_heads || xbc_stride < inner + 2 * groups * N ||
+        state_stride < (long long)n_heads * N * P)
+        return SIA_BAD_ARGUMENT;
+    const int channels = n_heads * N, share = n_heads / groups;
+    float* alpha = workspace;
+    float* kf = alpha + (size_t)n_tokens * channels;
+    float* raw_space = kf + (size_t)n_tokens * channels;
+    const int dt_col = row_stride - n_heads, b_col = inner, c_col = inner + groups * N;
+    dim3 pgrid(n_tokens, (channels + 255) / 256), pblock(256), fgrid(n_tokens, norm_groups), fblock(256);
+    bool raw = false;
+#define RUN(T)                                                                                                          \
+    do {                                                                                                                \
+        hipLaunchKernelGGL(ssd_prepare_kernel<T>, pgrid, pblock, 0, stream, (const T*)proj, row_stride, dt_col,         \
+                           (const T*)xbc, xbc_stride, b_col, dt_bias, a_log, alpha, kf, n_heads, N, share);             \
+        const int code = launch_recurrence(xbc, xbc_stride, c_col, 0, 0, -1, kf, share, alpha, norm_w, state,           \
+                                           state_stride, cu_q, slots, nullptr, n_seqs, max_q_len, n_heads, N, P, 1.f,   \
+                                           eps, dtype, raw_space, true, &raw, stream);                                  \
+        if (code) return code;                                                                                          \
+        hipLaunchKernelGGL(ssd_finish_kernel<T>, fgrid, fblock, 0, stream, raw_space, (const T*)proj, row_stride,       \
+                           (const T*)xbc, xbc_stride, d_skip, norm_w, (T*)out, inner, P, inner / norm_groups, eps);     \
+    } while (0)
+    if (dtype == SIA_F32) RUN(float);
+    else if (dtype == SIA_BF16) RUN(bf16_t);
+    else return SIA_BAD_ARGUMENT;
+#undef RUN
     return SIA_LAUNCH_CHECK();
 }

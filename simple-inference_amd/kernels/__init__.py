@@ -46,6 +46,24 @@ _SIGNATURES = {
                           _c_int, _c_ptr, _c_int, _c_ptr],
     "sia_gla_workspace": [_c_int, _c_int, _c_int, _c_int, _c_int, _c_int],
     "sia_moe_route": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr],
+    "sia_moe_route_ex": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
+                         _c_float, _c_ptr],
+    "sia_dyt_norm": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
+                     _c_int, _c_int, _c_int, _c_ptr],
+    "sia_causal_conv": [_c_ptr, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ll, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
+                        _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr],
+    "sia_hgrn2_workspace": [_c_int, _c_int, _c_int, _c_int],
+    "sia_hgrn2_scan": [_c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int,
+                       _c_int, _c_int, _c_int, _c_float, _c_int, _c_ptr, _c_ptr],
+    "sia_ssd_workspace": [_c_int, _c_int, _c_int, _c_int],
+    "sia_ssd_scan": [_c_ptr, _c_int, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ll, _c_ptr, _c_ptr,
+                     _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_ptr,
+                     _c_ptr],
+    "sia_latent_prepare": [_c_ptr, _c_int, _c_int, _c_ptr, _c_int, _c_ptr, _c_int, _c_int, _c_ptr, _c_ptr, _c_float,
+                           _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr, _c_int, _c_int,
+                           _c_ptr],
+    "sia_headwise_linear": [_c_ptr, _c_int, _c_int, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
+                            _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr],
     "sia_moe_gate_up": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr],
     "sia_moe_tiled_workspace": [_c_int, _c_int, _c_int, _c_int, _c_int],
     "sia_moe_tiled": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
@@ -185,6 +203,8 @@ class HipKernels:
         self.core.sia_sample_workspace_bytes.restype = ctypes.c_longlong
         self.core.sia_gla_workspace.restype = ctypes.c_longlong
         self.core.sia_moe_tiled_workspace.restype = ctypes.c_longlong
+        self.core.sia_hgrn2_workspace.restype = ctypes.c_longlong
+        self.core.sia_ssd_workspace.restype = ctypes.c_longlong
         self.tiled_experts = True        # many slots in bfloat16: experts' products on the matrix cores, slots sorted by expert
         self._attn_libs = {}
         # the short way to the current stream's handle, where this torch has it (a few microseconds less a launch)
@@ -493,9 +513,16 @@ class HipKernels:
             raise KernelError(f"head sizes {key_dim} x {value_dim} are outside what the recurrent kernel takes (up to {limit})")
 
     # -- mixture of experts ------------------------------------------------------------
-    def moe_route(self, h, router, top):
+    def moe_route(self, h, router, top, score="softmax", groups=None, scale=1.0):
         """The ``top`` experts of every row with the largest router logits ``h @ router^T`` (float; ties go to the
-        lower index) and the softmax over their logits alone: ``(ids [n, top] int32, weights [n, top] float32)``."""
+        lower index) and the softmax over their logits alone: ``(ids [n, top] int32, weights [n, top] float32)``.
+        ``score="sigmoid"``: the scores are the logits' sigmoids; with ``groups = (count, keep)`` only experts of the
+        ``keep`` groups (of ``count`` equal groups of neighbours) whose two largest scores sum highest can be chosen;
+        the weights are the chosen scores over their sum, times ``scale``."""
+        if score not in ("softmax", "sigmoid"):
+            raise KernelError(f"score must be 'softmax' or 'sigmoid', got {score!r}")
+        if score == "softmax" and (groups is not None or scale != 1.0):
+            raise KernelError("expert groups and a scale on the weights come with sigmoid scores")
         self._want(h, "router input")
         n, width = h.shape
         experts = router.shape[0]
@@ -504,9 +531,227 @@ class HipKernels:
             raise KernelError(f"router input must be float32 or bfloat16, is {h.dtype}")
         ids = torch.empty((n, top), dtype=torch.int32, device=h.device)
         weights = torch.empty((n, top), dtype=torch.float32, device=h.device)
-        self._check(self.core.sia_moe_route(_ptr(h), _ptr(router), _ptr(ids), _ptr(weights), n, width, experts, int(top),
-                                            _DT[h.dtype], self._stream()), "moe_route")
+        count, keep = (int(groups[0]), int(groups[1])) if groups else (0, 0)
+        if groups and (count <= 0 or experts % count or not 0 < keep <= count or top > experts // count * keep):
+            raise KernelError(f"{experts} experts in {count} groups of which {keep} are kept cannot give {top}")
+        if not 0 < top <= experts:
+            raise KernelError(f"top {top} is not between 1 and the number of experts {experts}")
+        self._check(self.core.sia_moe_route_ex(_ptr(h), _ptr(router), _ptr(ids), _ptr(weights), n, width, experts,
+                                               int(top), _DT[h.dtype], int(score == "sigmoid"), count, keep, float(scale),
+                                               self._stream()), "moe_route")
         return ids, weights
+
+    # -- norm without a statistic ---------------------------------------------------------
+    def dyt_norm(self, residual, delta, post, pre, out_dtype, rows=None):
+        """``x = residual (+ d)`` and ``norm(x)`` by a dynamic tanh, one kernel.  ``d`` is ``delta`` as it is, or with
+        ``post = (w, b, alpha, scale | None)`` the norm ``(tanh(alpha * delta) * w + b) * scale`` of it; ``pre`` holds
+        the same four terms of the norm whose rows are returned in ``out_dtype`` (None: only the sum is made).
+        Without ``rows`` the float residual is left updated; with ``rows`` (int32 indices) only those rows are
+        computed and the residual stays as it was."""
+        self._want(residual, "residual", torch.float32)
+        n, width = residual.shape
+        if out_dtype not in _DT:
+            raise KernelError(f"the norm's rows are float32 or bfloat16, not {out_dtype}")
+        if delta is not None:
+            self._want(delta, "delta", out_dtype, (n, width))
+        elif pre is None:
+            return None
+        terms = []
+        for t, what in ((post if delta is not None else None, "the delta's norm"), (pre, "norm")):
+            if t is None:
+                terms += [None, None, None, None]
+                continue
+            w, b, alpha, scale = t
+            self._want(w, f"{what} weight", torch.float32, (width,))
+            self._want(b, f"{what} bias", torch.float32, (width,))
+            self._want(alpha, f"{what} alpha", torch.float32, (1,))
+            if scale is not None:
+                self._want(scale, f"{what} scale", torch.float32, (width,))
+            terms += [w, b, alpha, scale]
+        n_out = n
+        if rows is not None:
+            self._want(rows, "rows", torch.int32)
+            n_out = rows.numel()
+        out = torch.empty((n_out, width), dtype=out_dtype, device=residual.device) if pre is not None else None
+        self._check(self.core.sia_dyt_norm(_ptr(residual), _ptr(delta), *(_ptr(t) for t in terms), _ptr(out), _ptr(rows),
+                                           n_out, width, _DT[out_dtype], self._stream()), "dyt_norm")
+        return out
+
+    # -- short convolution and recurrences with a state --------------------------------------
+    def _state_rows(self, state, ctx, least):
+        if state is None:
+            raise KernelError("a mixer with a state needs its state rows")
+        self._want(state, "state", torch.float32)
+        stride = state[0].numel()
+        if stride < least:
+            raise KernelError(f"a state row of {stride} floats does not hold {least}")
+        return stride
+
+    def _float_workspace(self, ctx, floats, device):
+        workspace = getattr(ctx, "recurrent_workspace", None)
+        if workspace is None or workspace.numel() < floats:
+            workspace = torch.empty((max(int(floats), 1),), dtype=torch.float32, device=device)
+            try:
+                ctx.recurrent_workspace = workspace
+            except AttributeError:
+                pass
+        return workspace
+
+    def causal_conv(self, proj, first_col, weight, bias, activation, ctx, state, state_offset):
+        """A causal convolution per channel over each sequence's tokens: ``out[t, c] = act(bias[c] + sum_j weight[c, j]
+        * u[t - (taps - 1) + j, c])`` with ``u`` the columns ``first_col .. first_col + channels - 1`` of ``proj``.  The
+        ``taps - 1`` inputs before a step's first token of a sequence are read from the sequence's state row at
+        ``state_offset`` (``[taps - 1, channels]`` floats, oldest first) and the row is left holding the last ones."""
+        self._want(proj, "projected rows")
+        n, width = proj.shape
+        channels, taps = weight.shape
+        if proj.dtype not in _DT or n != ctx.n_tokens:
+            raise KernelError(f"projected rows {proj.dtype} {tuple(proj.shape)} do not fit a step of {ctx.n_tokens} tokens")
+        self._want(weight, "convolution weight", torch.float32)
+        if bias is not None:
+            self._want(bias, "convolution bias", torch.float32, (channels,))
+        if activation not in (None, "silu"):
+            raise KernelError(f"the convolution's activation is silu or none, not {activation!r}")
+        if first_col < 0 or first_col + channels > width:
+            raise KernelError(f"columns {first_col} .. {first_col + channels} lie outside a row of {width}")
+        stride = self._state_rows(state, ctx, state_offset + channels * (taps - 1))
+        out = torch.empty((n, channels), dtype=proj.dtype, device=proj.device)
+        self._check(self.core.sia_causal_conv(
+            _ptr(proj), width, int(first_col), _ptr(weight), _ptr(bias), _ptr(state), stride, int(state_offset),
+            _ptr(ctx.cu_q), _ptr(ctx.seq_of_token), _ptr(ctx.state_slots), _ptr(out), n, ctx.n_seqs, ctx.max_q_len,
+            channels, taps, int(activation == "silu"), _DT[proj.dtype], self._stream()), "causal_conv")
+        return out
+
+    def ssd_scan(self, proj, xbc, dt_bias, a_log, d_skip, norm_weight, n_heads, head_dim, state_size, groups,
+                 norm_groups, eps, ctx, state):
+        """The state-space recurrence with a scalar decay per head over the step's runs of tokens.  ``proj`` rows are
+        ``[z (heads * head_dim) | ... | dt (heads)]``, ``xbc`` rows ``[x (heads * head_dim) | B (groups * state_size) |
+        C (groups * state_size)]``.  ``dt = softplus(dt + dt_bias)``; per head ``S <- exp(-exp(a_log) dt) S + dt B x^T``,
+        ``y = S^T C + d_skip x``; the result ``y * silu(z)`` is divided by the root mean square of each of
+        ``norm_groups`` equal parts and multiplied by ``norm_weight``.  The matrices ``[heads, state_size, head_dim]``
+        are the first floats of a sequence's state row."""
+        self._want(proj, "projected rows")
+        self._want(xbc, "convolved rows", proj.dtype)
+        n, width = proj.shape
+        inner = n_heads * head_dim
+        if proj.dtype not in _DT or n != ctx.n_tokens or xbc.shape[0] != n:
+            raise KernelError(f"rows {proj.dtype} {tuple(proj.shape)} do not fit a step of {ctx.n_tokens} tokens")
+        if width < inner + n_heads or xbc.shape[1] != inner + 2 * groups * state_size:
+            raise KernelError(f"rows of {width} and {xbc.shape[1]} do not hold {n_heads} heads of {head_dim} with "
+                              f"{groups} groups of {state_size}")
+        for t, what, size in ((dt_bias, "dt bias", n_heads), (a_log, "decay", n_heads), (d_skip, "skip", n_heads),
+                              (norm_weight, "norm weight", inner)):
+            self._want(t, what, torch.float32, (size,))
+        self.check_recurrent_geometry(state_size, head_dim)
+        if n_heads % groups or inner % norm_groups:
+            raise KernelError(f"{n_heads} heads of {head_dim} do not split into {groups} groups and {norm_groups} parts")
+        stride = self._state_rows(state, ctx, n_heads * state_size * head_dim)
+        out = torch.empty((n, inner), dtype=proj.dtype, device=proj.device)
+        workspace = self._float_workspace(ctx, self.core.sia_ssd_workspace(n, n_heads, state_size, head_dim), proj.device)
+        self._check(self.core.sia_ssd_scan(
+            _ptr(proj), width, _ptr(xbc), xbc.shape[1], _ptr(dt_bias), _ptr(a_log), _ptr(d_skip), _ptr(norm_weight),
+            _ptr(state), stride, _ptr(ctx.cu_q), _ptr(ctx.state_slots), _ptr(out), n, ctx.n_seqs, ctx.max_q_len, n_heads,
+            head_dim, state_size, groups, norm_groups, float(eps), _DT[proj.dtype], _ptr(workspace), self._stream()),
+            "ssd_scan")
+        return out
+
+    def hgrn2_scan(self, proj, f_bias, lower, norm_weight, n_heads, key_dim, value_dim, eps, ctx, state):
+        """The gated linear recurrence whose forget gate also decides what is written.  ``proj`` rows are ``[q | f | v]``
+        (``heads * key_dim``, the same, ``heads * value_dim``) and are used up (the q columns are overwritten).
+        ``f = lower + (1 - lower) * sigmoid(f + f_bias)``; per head ``S <- diag(f) S + (1 - f) v^T``, ``o = S^T silu(q)``;
+        every head's ``o`` is divided by its root mean square and multiplied by ``norm_weight``.  The state rows are
+        ``[heads, key_dim, value_dim]`` floats."""
+        self._want(proj, "projected rows")
+        n, width = proj.shape
+        qk = n_heads * key_dim
+        if proj.dtype not in _DT or n != ctx.n_tokens or width != 2 * qk + n_heads * value_dim:
+            raise KernelError(f"projected rows {proj.dtype} {tuple(proj.shape)} do not fit {ctx.n_tokens} tokens of "
+                              f"{n_heads} heads of {key_dim} and {value_dim}")
+        self._want(f_bias, "forget bias", torch.float32, (qk,))
+        self._want(lower, "lower bound", torch.float32, (qk,))
+        self._want(norm_weight, "output norm weight", torch.float32, (value_dim,))
+        self.check_recurrent_geometry(key_dim, value_dim)
+        if state is None or tuple(state.shape[1:]) != (n_heads, key_dim, value_dim):
+            raise KernelError(f"state rows are not [{n_heads}, {key_dim}, {value_dim}]")
+        self._state_rows(state, ctx, qk * value_dim)
+        out = torch.empty((n, n_heads * value_dim), dtype=proj.dtype, device=proj.device)
+        workspace = self._float_workspace(ctx, self.core.sia_hgrn2_workspace(n, n_heads, key_dim, value_dim), proj.device)
+        self._check(self.core.sia_hgrn2_scan(
+            _ptr(proj), width, _ptr(f_bias), _ptr(lower), _ptr(norm_weight), _ptr(state), _ptr(ctx.cu_q),
+            _ptr(ctx.state_slots), _ptr(out), n, ctx.n_seqs, ctx.max_q_len, n_heads, key_dim, value_dim, float(eps),
+            _DT[proj.dtype], _ptr(workspace), self._stream()), "hgrn2_scan")
+        return out
+
+    # -- latent attention ---------------------------------------------------------------------
+    def _rotation_tables(self, rotary_dim, cos, sin, ctx_or_len):
+        if not rotary_dim:
+            return None, None
+        for t, what in ((cos, "cos table"), (sin, "sin table")):
+            self._want(t, what, torch.float32)
+            if t.shape[1] != rotary_dim // 2 or t.shape[0] <= ctx_or_len - 1:
+                raise KernelError(f"{what} {tuple(t.shape)} does not cover position {ctx_or_len - 1} with "
+                                  f"{rotary_dim // 2} pairs")
+        return cos, sin
+
+    def latent_prepare(self, proj, q_rank, q_gain, kv_rank, kv_gain, rot_dim, rotary_dim, cos, sin, eps, ctx, cache,
+                       page_dim=None):
+        """From projected rows ``[a_q (q_rank) | a (kv_rank) | b (rot_dim)]``: returns ``rms(a_q) * q_gain`` and, if
+        ``kv_rank`` is not 0, writes ``[rms(a) * kv_gain | rotate(b)]`` as the position's key row and ``rms(a) *
+        kv_gain`` as its value into the pages (one key/value head; rows ``page_dim`` wide if given).  The rotation
+        turns neighbouring pairs of the first ``rotary_dim`` elements of ``b``."""
+        self._want(proj, "projected rows")
+        n, width = proj.shape
+        if proj.dtype not in _DT or n != ctx.n_tokens or width != q_rank + (kv_rank + rot_dim if kv_rank else 0):
+            raise KernelError(f"projected rows {proj.dtype} {tuple(proj.shape)} do not fit {ctx.n_tokens} tokens of "
+                              f"{q_rank} + {kv_rank} + {rot_dim} columns")
+        self._want(q_gain, "query latent gain", torch.float32, (q_rank,))
+        cq = torch.empty((n, q_rank), dtype=proj.dtype, device=proj.device)
+        table = k_pages = v_pages = None
+        page_size = key_width = value_rows = 0
+        if kv_rank:
+            self._want(kv_gain, "latent gain", torch.float32, (kv_rank,))
+            cos, sin = self._rotation_tables(rotary_dim, cos, sin, ctx.max_kv_len)
+            key_width = page_dim or (kv_rank + rot_dim)
+            value_rows = page_dim or kv_rank
+            k_pages, v_pages, table, page_size = cache.k_pages, cache.v_pages, cache.block_table, cache.page_size
+            self._check_pages(k_pages, v_pages, table, page_size, 1, key_width, proj.dtype, ctx, value_rows)
+        self._check(self.core.sia_latent_prepare(
+            _ptr(proj), width, q_rank, _ptr(q_gain), kv_rank, _ptr(kv_gain), rot_dim, rotary_dim if kv_rank else 0,
+            _ptr(cos) if kv_rank else None, _ptr(sin) if kv_rank else None, float(eps), _ptr(ctx.positions),
+            _ptr(ctx.seq_of_token), _ptr(table), table.shape[1] if table is not None else 0, _ptr(k_pages),
+            _ptr(v_pages), page_size, key_width, value_rows, _ptr(cq), n, _DT[proj.dtype], self._stream()),
+            "latent_prepare")
+        return cq
+
+    def headwise_linear(self, x, w, in_stride, out_stride, tail=0, rotation=None):
+        """A product per head: ``y[n, h, :out] = w[h] x[n, h, :in]`` for ``w [heads, out, in]``, ``x`` rows holding
+        ``in_stride`` elements a head and ``y`` rows ``out_stride``.  The ``tail`` elements behind a head's inputs are
+        copied behind its outputs, their first ``rotary_dim`` elements turned in neighbouring pairs by ``rotation =
+        (rotary_dim, cos, sin, positions)``; what is left of a head's ``out_stride`` is zero."""
+        self._want(x, "headwise input")
+        self._want(w, "headwise weights", x.dtype)
+        if x.dtype not in _DT or w.dim() != 3:
+            raise KernelError(f"a product per head takes float32 or bfloat16 rows and weights [heads, out, in]")
+        n, width = x.shape
+        heads, out_dim, in_dim = w.shape
+        if width != heads * in_stride or in_dim + tail > in_stride or out_dim + tail > out_stride:
+            raise KernelError(f"rows of {width} do not hold {heads} heads of {in_stride}, or {in_dim} + {tail} inputs and "
+                              f"{out_dim} + {tail} outputs do not fit strides {in_stride} and {out_stride}")
+        rotary_dim, cos, sin, positions = rotation if (rotation is not None and tail) else (0, None, None, None)
+        if rotary_dim:
+            if rotary_dim > tail or rotary_dim % 2:
+                raise KernelError(f"a rotation of {rotary_dim} elements does not fit a tail of {tail}")
+            self._want(positions, "positions", torch.int32, (n,))
+            for t, what in ((cos, "cos table"), (sin, "sin table")):
+                self._want(t, what, torch.float32)
+                if t.shape[1] != rotary_dim // 2:
+                    raise KernelError(f"{what} {tuple(t.shape)} does not hold {rotary_dim // 2} pairs")
+        y = torch.empty((n, heads * out_stride), dtype=x.dtype, device=x.device)
+        self._check(self.core.sia_headwise_linear(
+            _ptr(x), width, in_stride, _ptr(w), _ptr(y), heads * out_stride, out_stride, n, heads, in_dim, out_dim,
+            int(tail), int(rotary_dim), _ptr(cos) if rotary_dim else None, _ptr(sin) if rotary_dim else None,
+            _ptr(positions) if rotary_dim else None, _DT[x.dtype], self._stream()), "headwise_linear")
+        return y
 
     def moe_experts(self, h, w_gate_up, w_down, ids, weights, shared=None, shared_gate=None):
         """``sum_k weights[n, k] * expert_{ids[n, k]}(h[n])`` with ``expert_e(x) = W2_e (silu(Wg_e x) * (Wu_e x))``,
