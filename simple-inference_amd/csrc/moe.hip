@@ -62,7 +62,7 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const T* __restrict__ h,
             int which = 0x7fffffff;
             for (int g = lane; g < n_groups; g += SIA_WAVE) {
                 const float z = group_s[g];
-                if (z > best) { best = z; which = g; }
+                if (z != INFINITY && z > best) { best = z; which = g; }      // a kept group is out of the next rounds
             }
 #pragma unroll
             for (int off = SIA_WAVE / 2; off > 0; off >>= 1) {

@@ -48,7 +48,7 @@ def _mixer(cfg: FamepelConfig, m, p: str) -> PartSpec:
         "value_head_dim": m.vdim, "q_rank": m.q_rank, "kv_rank": m.kv_rank, "scale": m.scale,
         "norm_eps": cfg.norm_eps, "sink": True, "kv_from_layer": m.kv_from,
         "position": {"kind": "rope", "params": {"rotary_dim": m.rot.dims, "theta": m.rot.base, "scaling": scaling,
-                                                "pairing": "interleaved"}},
+                                                "pairing": "interleaved", "angles": "float64"}},
     }, names, role="mixer")
 
 

@@ -69,7 +69,8 @@ def yarn_inv_freq(rotary_dim: int, theta: float, scaling) -> tuple:
 @register_position_encoding("rope")
 class RotaryEncoding:
     """params: rotary_dim, theta, scaling (dict or None), and optionally pairing ("half", the default, or
-    "interleaved")."""
+    "interleaved") and angles ("float32", the default: positions times frequencies as float32 products, or "float64":
+    frequencies and angles in float64 on the host, the tables rounded once)."""
 
     def __init__(self, params, env):
         self.rotary_dim = int(params["rotary_dim"])
@@ -80,6 +81,9 @@ class RotaryEncoding:
         self.pairing = str(params.get("pairing", "half"))
         if self.pairing not in ("half", "interleaved"):
             raise ValueError(f"pairing must be 'half' or 'interleaved', got {self.pairing!r}")
+        self.angles = str(params.get("angles", "float32"))
+        if self.angles not in ("float32", "float64"):
+            raise ValueError(f"angles must be 'float32' or 'float64', got {self.angles!r}")
         self.max_positions = int(env.max_positions)
         self.device = env.device
         self._tables = None
@@ -96,6 +100,8 @@ class RotaryEncoding:
             amplitude = 1.0
             if self.scaling is not None and self.scaling.get("rope_type") == "yarn":
                 inv_freq, amplitude = yarn_inv_freq(self.rotary_dim, self.theta, self.scaling)
+            elif self.angles == "float64" and self.scaling is None:
+                inv_freq = self.theta ** (-torch.arange(0, self.rotary_dim, 2, dtype=torch.float64) / self.rotary_dim)
             else:
                 inv_freq = rotary_inv_freq(self.rotary_dim, self.theta, self.scaling)
             # the ramp form's angles are taken in float64 on the host and the tables rounded once

@@ -45,12 +45,20 @@ def causal_conv(u, w, b):
     return out
 
 
-def mamba2(h, T, p, m, eps):
+def mamba2_inputs(h, T, p, m):
+    """The mixer's projection and convolution: ``z [n, inner]``, the convolved ``[x | B | C]`` rows and the raw step
+    sizes ``[n, heads]``."""
     heads, vdim, N, G = m["heads"], m["vdim"], m["state"], m["groups"]
-    inner, n = heads * vdim, h.shape[0]
+    inner = heads * vdim
     proj = h @ _t(T, p + ".in").T
     z, xbc, dt = proj[:, :inner], proj[:, inner:2 * inner + 2 * G * N], proj[:, 2 * inner + 2 * G * N:]
-    xbc = silu(causal_conv(xbc, _t(T, p + ".conv"), _t(T, p + ".conv.b")))
+    return z, silu(causal_conv(xbc, _t(T, p + ".conv"), _t(T, p + ".conv.b"))), dt
+
+
+def state_space(z, xbc, dt, T, p, m, eps):
+    """The recurrence over convolved rows, the gate and the norm in parts: ``[n, inner]``."""
+    heads, vdim, N, G = m["heads"], m["vdim"], m["state"], m["groups"]
+    inner, n = heads * vdim, z.shape[0]
     x = xbc[:, :inner].reshape(n, heads, vdim)
     B = xbc[:, inner:inner + G * N].reshape(n, G, N)
     C = xbc[:, inner + G * N:].reshape(n, G, N)
@@ -66,8 +74,12 @@ def mamba2(h, T, p, m, eps):
             y[t, hd] = S.T @ C[t, g] + D[hd] * x[t, hd]
     y = y.reshape(n, inner) * silu(z)
     parts = m["norm_groups"]
-    y = rms(y.reshape(n, parts, inner // parts), eps).reshape(n, inner) * _t(T, p + ".norm")
-    return y @ _t(T, p + ".o").T
+    return rms(y.reshape(n, parts, inner // parts), eps).reshape(n, inner) * _t(T, p + ".norm")
+
+
+def mamba2(h, T, p, m, eps):
+    z, xbc, dt = mamba2_inputs(h, T, p, m)
+    return state_space(z, xbc, dt, T, p, m, eps) @ _t(T, p + ".o").T
 
 
 # ---------------------------------------------------------------------------------------------------------
