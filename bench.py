@@ -26,6 +26,9 @@ weights): decode at batch 8 and 1 over 2,048-token contexts and the prefill of 2
 fraction of the HBM or matrix-core roofline, in one JSON line of its own kind.
 ``--workload mogisun`` does the same for the Mogisun design: a model of softmax-attention layers with dense
 feed-forwards and a model of linear-attention layers with routed experts, each beside the Llama model.
+``--workload famepel`` does the same for the Famepel design: a model of each of its three mixers (state-space,
+forget-gate recurrence, latent attention), all with grouped experts, beside the Mogisun model of linear-attention
+layers with routed experts and the Llama model.
 
 The engine runs on one GPU; asked for more it says so and exits with 2.
 """
@@ -78,10 +81,11 @@ def parse_args(argv=None):
     ap.add_argument("--temperature", type=float, default=0.0, help="sampling of the decode measurement (0: greedy)")
     ap.add_argument("--top-k", type=int, default=0)
     ap.add_argument("--top-p", type=float, default=1.0)
-    ap.add_argument("--workload", default="decode", choices=["decode", "continuous", "shared-prefix", "feduzen", "mogisun"])
+    ap.add_argument("--workload", default="decode", choices=["decode", "continuous", "shared-prefix", "feduzen", "mogisun", "famepel"])
     ap.add_argument("--shapes", default="1b,3b,8b", help="--workload feduzen: which layer sizes, comma separated")
-    ap.add_argument("--models", default=None, help="--workload feduzen or mogisun: which of the models to run "
-                    "(feduzen,llama; mogisun-attention,mogisun-linear,llama)")
+    ap.add_argument("--models", default=None, help="--workload feduzen, mogisun or famepel: which of the models to run "
+                    "(feduzen,llama; mogisun-attention,mogisun-linear,llama; famepel-ssm,famepel-hgrn,famepel-latent,"
+                    "mogisun-linear,llama)")
     ap.add_argument("--max-running", type=int, default=64, help="request slots of the stream workloads")
     return ap.parse_args(argv)
 
@@ -425,22 +429,18 @@ def mogisun_config_like(llama_cfg, layers, kind):
             "layers": [json.loads(json.dumps(layer)) for _ in range(layers)]}
 
 
-def mogisun_workload(args):
-    """Decode and prefill of the Mogisun design (its two kinds of layer, each alone) beside the Llama model at equal
-    layer sizes."""
+def measure_beside(args, models, wanted):
+    """Decode at batch 8 and 1 and the prefill of every wanted model of ``models(llama_cfg, layers)`` at every shape."""
     from simple_inference_amd import Engine, EngineConfig, preset
 
     layers = args.layers or 8
-    dt_name = "bf16" if args.dtype == "bfloat16" else "fp32"
     context, T = args.context, args.prefill_tokens
     total_len = max(context + args.warmup + args.steps + decode_allowance(max(2048, T), 8, context), T + 2)
-    wanted = (args.models or "mogisun-attention,mogisun-linear,llama").split(",")
     out = {}
     for shape in [x for x in args.shapes.split(",") if x]:
         llama = preset(FEDUZEN_SHAPES[shape])
         llama["num_hidden_layers"] = layers
-        for model, cfg in (("mogisun-attention", mogisun_config_like(llama, layers, "attention")),
-                           ("mogisun-linear", mogisun_config_like(llama, layers, "linear")), ("llama", llama)):
+        for model, cfg in models(llama, layers):
             if model not in wanted:
                 continue
             ecfg = EngineConfig(max_running=8, max_seq_len=max(4096, -(-total_len // 1024) * 1024), dtype=args.dtype,
@@ -457,11 +457,76 @@ def mogisun_workload(args):
             out.setdefault(shape, {})[model] = row
             del engine
             torch.cuda.empty_cache()
+    return out
+
+
+def mogisun_workload(args):
+    """Decode and prefill of the Mogisun design (its two kinds of layer, each alone) beside the Llama model at equal
+    layer sizes."""
+    layers = args.layers or 8
+    dt_name = "bf16" if args.dtype == "bfloat16" else "fp32"
+    out = measure_beside(args, lambda llama, n: (("mogisun-attention", mogisun_config_like(llama, n, "attention")),
+                                                 ("mogisun-linear", mogisun_config_like(llama, n, "linear")),
+                                                 ("llama", llama)),
+                         (args.models or "mogisun-attention,mogisun-linear,llama").split(","))
     line = {"metric": "Mogisun beside Llama at equal layer sizes: decode tok/s (batch 8, 1) and prefill tok/s",
             "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "dtype": dt_name,
             "data": "synthetic (seeded random weights and uniform-random token ids)",
-            "config": {"layers": layers, "context": context, "prefill_tokens": T, "shapes": FEDUZEN_SHAPES,
+            "config": {"layers": layers, "context": args.context, "prefill_tokens": args.prefill_tokens,
+                       "shapes": FEDUZEN_SHAPES,
                        "mogisun-attention": "softmax attention with its gates, norms and temperature, dense SwiGLU",
+                       "mogisun-linear": "gated linear attention, 8 experts of ff/4 (2 a token) and a shared one of ff/2"},
+            "shapes": out}
+    print(json.dumps(line), flush=True)
+    return 0
+
+
+def famepel_config_like(llama_cfg, layers, kind):
+    """A Famepel config.json with the width, head count, head width and feed-forward size of a Llama one; every layer
+    has the same mixer and eight experts of half the feed-forward size in four groups, two groups kept and two
+    experts a token (as many active feed-forward weights as the dense layer has).  ``ssm``: as many heads of the
+    same width, a state of that size too, one group, a convolution of four taps.  ``hgrn``: as many heads, keys and
+    values of the head width.  ``latent``: as many heads, a latent of 192 and a shared rotated key part of 64 (a
+    cached row of 256 elements whatever the number of heads), queries through a latent of half the width."""
+    dim, heads, width = llama_cfg["head_dim"], llama_cfg["num_attention_heads"], llama_cfg["hidden_size"]
+    if kind == "ssm":
+        mixer = {"type": "mamba2", "mixer": {"conv": 4, "groups": 1, "heads": heads, "norm_groups": 1, "state": dim,
+                                             "vdim": dim}}
+    elif kind == "hgrn":
+        mixer = {"type": "hgrn2", "mixer": {"dim": dim, "heads": heads, "vdim": dim}}
+    else:
+        mixer = {"type": "latent_attention",
+                 "mixer": {"dim": dim, "heads": heads, "kv_rank": 192, "q_rank": width // 2, "rot_dim": 64, "vdim": dim,
+                           "scale": (dim + 64) ** -0.5,
+                           "rot": {"base": llama_cfg["rope_theta"], "dims": 64,
+                                   "scaling": {"factor": 8.0, "original": 8192, "fast": 32.0, "slow": 1.0}}}}
+    mlp = {"kind": "moe", "expert": {"ff": llama_cfg["intermediate_size"] // 2},
+           "router": {"experts": 8, "top": 2, "scale": 2.5, "groups": {"count": 4, "keep": 2}}}
+    return {"architecture": "Famepel", "vocab": llama_cfg["vocab_size"], "width": width,
+            "norm": {"eps": llama_cfg["rms_norm_eps"]}, "embedding": {"scale": 1.0},
+            "layers": [json.loads(json.dumps(dict(mixer, mlp=mlp))) for _ in range(layers)]}
+
+
+def famepel_workload(args):
+    """Decode and prefill of the Famepel design (each of its three mixers alone, with its experts) beside the Mogisun
+    model of linear-attention layers with routed experts and the Llama model at equal layer sizes."""
+    layers = args.layers or 8
+    dt_name = "bf16" if args.dtype == "bfloat16" else "fp32"
+    out = measure_beside(args, lambda llama, n: (("famepel-ssm", famepel_config_like(llama, n, "ssm")),
+                                                 ("famepel-hgrn", famepel_config_like(llama, n, "hgrn")),
+                                                 ("famepel-latent", famepel_config_like(llama, n, "latent")),
+                                                 ("mogisun-linear", mogisun_config_like(llama, n, "linear")),
+                                                 ("llama", llama)),
+                         (args.models or "famepel-ssm,famepel-hgrn,famepel-latent,mogisun-linear,llama").split(","))
+    line = {"metric": "Famepel beside Mogisun and Llama at equal layer sizes: decode tok/s (batch 8, 1) and prefill tok/s",
+            "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "dtype": dt_name,
+            "data": "synthetic (seeded random weights and uniform-random token ids)",
+            "config": {"layers": layers, "context": args.context, "prefill_tokens": args.prefill_tokens,
+                       "shapes": FEDUZEN_SHAPES,
+                       "famepel-*": "dynamic-tanh norms around every sublayer; 8 experts of ff/2 in 4 groups, 2 kept, 2 a token",
+                       "famepel-ssm": "state-space mixer: heads of the head width, state of that size, 4 taps",
+                       "famepel-hgrn": "forget-gate recurrence: heads with keys and values of the head width",
+                       "famepel-latent": "latent attention: latent 192 + rotated 64 cached, queries through width/2",
                        "mogisun-linear": "gated linear attention, 8 experts of ff/4 (2 a token) and a shared one of ff/2"},
             "shapes": out}
     print(json.dumps(line), flush=True)
@@ -538,6 +603,8 @@ def main(argv=None):
         return feduzen_workload(args)
     if args.workload == "mogisun":
         return mogisun_workload(args)
+    if args.workload == "famepel":
+        return famepel_workload(args)
     if args.workload != "decode":
         return stream_workload(args)
     points = [int(p) for p in args.points.split(",") if p]
