@@ -446,7 +446,7 @@ __global__ __launch_bounds__(DEC_WAVES* SIA_WAVE) void attn_decode_kernel(
     const int* __restrict__ block_table, int table_width, const int* __restrict__ cu_q,
     const int* __restrict__ kv_len, float* __restrict__ ws_acc, float* __restrict__ ws_ml,
     bf16_t* __restrict__ out, int n_heads, int n_kv, int ps_log2, float scale, int window, int chunk,
-    const float* __restrict__ sinks, int max_splits, int mode) {
+    const float* __restrict__ sinks, int max_splits, int mode, int kv_share) {
     const bool fold = mode == DEC_FOLD, spread = mode == DEC_SPREAD;
     static_assert(DEC_WAVES == 4, "merge_waves merges four runs");
     extern __shared__ float lds[];  // [runs of the workgroup][group][HD + 2]
@@ -505,7 +505,7 @@ __global__ __launch_bounds__(DEC_WAVES* SIA_WAVE) void attn_decode_kernel(
     if (first < end) {  // wave-uniform
         const int w_lo = max(lo_all, first * TILE), w_hi = min(pos, end * TILE - 1);
         const int lo[1] = {r < group ? w_lo : 1}, hi[1] = {r < group ? w_hi : 0};
-        attend_range<1>(qf, kp, vp, table, table_width, ps_log2, n_kv, hk, w_lo, w_hi, lo, hi, scale, sm, acc,
+        attend_range<1>(qf, kp, vp, table, table_width, ps_log2, n_kv / kv_share, hk / kv_share, w_lo, w_hi, lo, hi, scale, sm, acc,
                         at_run_ends);
     }
     while (at_run_ends.done < mine_n - 1) at_run_ends.pass();  // runs without tiles of their own
@@ -1043,16 +1043,19 @@ SIA_EXPORT long long sia_attn_decode_workspace(int n_seqs, int n_heads, int n_kv
 // sia_attn_decode_workspace(.., 0) and (.., 1) floats (neither is read before it is written).
 // chunk > 0: a query sees only its own block of chunk positions (max_splits then from min(window, chunk), whichever
 // are given); sinks: one float per query head that joins its softmax's denominator, or null.
-SIA_EXPORT int sia_attn_decode_ex(const void* q, int q_row_stride, const void* k_pages, const void* v_pages,
-                                  const int* block_table, int table_width, const int* cu_q, const int* kv_len,
-                                  void* out, float* ws_acc, float* ws_ml, int n_seqs, int n_heads, int n_kv,
-                                  int page_size, float scale, int window, int chunk, const float* sinks,
-                                  int max_splits, hipStream_t stream) {
+// kv_share > 1: the pages hold n_kv / kv_share key/value heads, and each is read by kv_share of the launch's n_kv
+// groups of query heads (more than 16 query heads on one key/value head are dealt out as several groups).
+SIA_EXPORT int sia_attn_decode_shared(const void* q, int q_row_stride, const void* k_pages, const void* v_pages,
+                                      const int* block_table, int table_width, const int* cu_q, const int* kv_len,
+                                      void* out, float* ws_acc, float* ws_ml, int n_seqs, int n_heads, int n_kv,
+                                      int kv_share, int page_size, float scale, int window, int chunk,
+                                      const float* sinks, int max_splits, hipStream_t stream) {
     if (n_seqs <= 0) return 0;
     const int ps_log2 = log2_exact(page_size);
     const int n_splits = max_splits;
-    if (ps_log2 < 3 || n_kv <= 0 || n_heads % n_kv || n_heads / n_kv > 16 || n_splits <= 0 ||
-        n_splits > DEC_MAX_SPLITS || n_kv > 65535 || n_seqs > 65535 || q_row_stride % 8 || table_width <= 0)
+    if (ps_log2 < 3 || n_kv <= 0 || n_heads % n_kv || n_heads / n_kv > 16 || n_splits <= 0 || kv_share <= 0 ||
+        n_kv % kv_share || n_splits > DEC_MAX_SPLITS || n_kv > 65535 || n_seqs > 65535 || q_row_stride % 8 ||
+        table_width <= 0)
         return SIA_BAD_ARGUMENT;
     const DecodeMode mode = decode_mode(n_seqs, n_heads, n_kv, n_splits);
     if ((sia_attn_decode_workspace(n_seqs, n_heads, n_kv, n_splits, 0) && !ws_acc) ||
@@ -1079,12 +1082,23 @@ SIA_EXPORT int sia_attn_decode_ex(const void* q, int q_row_stride, const void* k
     hipLaunchKernelGGL(attn_decode_kernel, grid, dim3((mode == DEC_SPREAD ? 1 : DEC_WAVES) * SIA_WAVE),
                        mode == DEC_SPREAD ? 0 : lds_bytes, stream, (const bf16_t*)q, q_row_stride,
                        (const bf16_t*)k_pages, (const bf16_t*)v_pages, block_table, table_width, cu_q, kv_len, ws_acc,
-                       ws_ml, (bf16_t*)out, n_heads, n_kv, ps_log2, scale, window, chunk, sinks, n_splits, (int)mode);
+                       ws_ml, (bf16_t*)out, n_heads, n_kv, ps_log2, scale, window, chunk, sinks, n_splits, (int)mode,
+                       kv_share);
     if (mode == DEC_SPREAD || (mode == DEC_PLAIN && n_splits > 1))
         hipLaunchKernelGGL(attn_decode_combine_kernel, dim3(n_heads, n_seqs), dim3(SIA_WAVE), 0, stream, ws_acc,
                            ws_ml, cu_q, kv_len, (bf16_t*)out, n_heads, n_splits, window, chunk, sinks,
                            mode == DEC_SPREAD ? 1 : 0);
     return SIA_LAUNCH_CHECK();
+}
+
+SIA_EXPORT int sia_attn_decode_ex(const void* q, int q_row_stride, const void* k_pages, const void* v_pages,
+                                  const int* block_table, int table_width, const int* cu_q, const int* kv_len,
+                                  void* out, float* ws_acc, float* ws_ml, int n_seqs, int n_heads, int n_kv,
+                                  int page_size, float scale, int window, int chunk, const float* sinks,
+                                  int max_splits, hipStream_t stream) {
+    return sia_attn_decode_shared(q, q_row_stride, k_pages, v_pages, block_table, table_width, cu_q, kv_len, out,
+                                  ws_acc, ws_ml, n_seqs, n_heads, n_kv, 1, page_size, scale, window, chunk, sinks,
+                                  max_splits, stream);
 }
 
 SIA_EXPORT int sia_attn_decode(const void* q, int q_row_stride, const void* k_pages, const void* v_pages,

@@ -134,11 +134,15 @@ __device__ __forceinline__ float row16_sum(float v) {
 // that the walk never waits for memory.  Outputs go to the float workspace; the norm is the finishing kernel's.
 #define GLA_WALK_TOKENS 32
 #define GLA_WALK_THREADS 256
-template <int ROWS, int GLA_WALK_COLS>
+// KF: what is written (k) comes as floats [tokens, heads, D] from ``k_f32``, as the decays do, not as columns of the
+// rows.  ``q_share`` neighbouring heads read the same q columns; a sequence's matrices begin ``state_stride`` floats
+// after the sequence before it.
+template <int ROWS, int GLA_WALK_COLS, bool KF>
 __global__ __launch_bounds__(GLA_WALK_THREADS) void gla_walk_kernel(
     const bf16_t* __restrict__ proj, int row_stride, int q_col, int k_col, int v_col, const float* __restrict__ alpha,
-    float* __restrict__ state, const int* __restrict__ cu_q, const int* __restrict__ slots, int n_heads, int D, int Dv,
-    float q_scale, float* __restrict__ raw_out) {
+    const float* __restrict__ k_f32, int q_share, float* __restrict__ state, long long state_stride,
+    const int* __restrict__ cu_q, const int* __restrict__ slots, int n_heads, int D, int Dv, float q_scale,
+    float* __restrict__ raw_out) {
     extern __shared__ float lds[];
     constexpr int TB = GLA_WALK_TOKENS, C = GLA_WALK_COLS, threads = GLA_WALK_THREADS;
     constexpr int slice = threads / 16 * C;      // columns a workgroup
@@ -155,7 +159,7 @@ __global__ __launch_bounds__(GLA_WALK_THREADS) void gla_walk_kernel(
     auto place = [](int d) { const int r = d / ROWS, i = d % ROWS; return (i / 4) * 64 + r * 4 + i % 4; };
     for (int i = tid; i < 3 * TB * Dp; i += threads) lds[i] = 0.f;
     const int jl = (tid / 16) * C, r = tid % 16;      // this lane's first column inside the slice, and its rows
-    float* S_mem = state + ((size_t)slots[seq] * n_heads + head) * D * Dv;
+    float* S_mem = state + (size_t)slots[seq] * state_stride + (size_t)head * D * Dv;
     float S[C][ROWS];
 #pragma unroll
     for (int c = 0; c < C; ++c)
@@ -165,25 +169,28 @@ __global__ __launch_bounds__(GLA_WALK_THREADS) void gla_walk_kernel(
             S[c][i] = (j < Dv && d < D) ? S_mem[(size_t)d * Dv + j] : 0.f;
         }
     const int d8 = D / 8, d4 = D / 4;
+    const int q_at = q_col + (head / q_share) * D, k_at = k_col + (head / q_share) * D;
     // What is on its way from memory is held in named registers, and the two steps below are written out piece by
     // piece: arrays indexed in loops ended up in scratch memory here, and a wave then waited for every piece twice.
     static_assert(TB * slice / threads == 4, "four values a thread and block");
     uint4 rq0, rq1, rq2, rq3, rk0, rk1, rk2, rk3;
     float4 ra0, ra1, ra2, ra3, ra4, ra5, ra6, ra7;
+    float4 rf0, rf1, rf2, rf3, rf4, rf5, rf6, rf7;
     float rv0, rv1, rv2, rv3;
     // pieces beyond the block's end repeat its last piece (every load is issued, none is conditional)
 #define GLA_REQ_QK(i, Q, K)                                                                          \
     do {                                                                                             \
         const int idx = min(tid + (i) * threads, rnt * d8 - 1);                                       \
-        const bf16_t* row = proj + (size_t)(rt0 + idx / d8) * row_stride + head * D + (idx % d8) * 8; \
-        Q = *reinterpret_cast<const uint4*>(row + q_col);                                            \
-        K = *reinterpret_cast<const uint4*>(row + k_col);                                            \
+        const bf16_t* row = proj + (size_t)(rt0 + idx / d8) * row_stride + (idx % d8) * 8;            \
+        Q = *reinterpret_cast<const uint4*>(row + q_at);                                             \
+        if constexpr (!KF) K = *reinterpret_cast<const uint4*>(row + k_at);                          \
     } while (0)
-#define GLA_REQ_A(i, A)                                                                              \
+#define GLA_REQ_F(i, A, SRC)                                                                         \
     do {                                                                                             \
         const int idx = min(tid + (i) * threads, rnt * d4 - 1);                                       \
-        A = *reinterpret_cast<const float4*>(alpha + ((size_t)(rt0 + idx / d4) * n_heads + head) * D + (idx % d4) * 4); \
+        A = *reinterpret_cast<const float4*>(SRC + ((size_t)(rt0 + idx / d4) * n_heads + head) * D + (idx % d4) * 4); \
     } while (0)
+#define GLA_REQ_A(i, A) GLA_REQ_F(i, A, alpha)
 #define GLA_REQ_V(i, V)                                                                              \
     do {                                                                                             \
         const int idx = min(tid + (i) * threads, rnt * slice - 1);                                    \
@@ -196,6 +203,10 @@ __global__ __launch_bounds__(GLA_WALK_THREADS) void gla_walk_kernel(
         GLA_REQ_QK(0, rq0, rk0); GLA_REQ_QK(1, rq1, rk1); GLA_REQ_QK(2, rq2, rk2); GLA_REQ_QK(3, rq3, rk3); \
         GLA_REQ_A(0, ra0); GLA_REQ_A(1, ra1); GLA_REQ_A(2, ra2); GLA_REQ_A(3, ra3);                  \
         GLA_REQ_A(4, ra4); GLA_REQ_A(5, ra5); GLA_REQ_A(6, ra6); GLA_REQ_A(7, ra7);                  \
+        if constexpr (KF) {                                                                          \
+            GLA_REQ_F(0, rf0, k_f32); GLA_REQ_F(1, rf1, k_f32); GLA_REQ_F(2, rf2, k_f32); GLA_REQ_F(3, rf3, k_f32); \
+            GLA_REQ_F(4, rf4, k_f32); GLA_REQ_F(5, rf5, k_f32); GLA_REQ_F(6, rf6, k_f32); GLA_REQ_F(7, rf7, k_f32); \
+        }                                                                                            \
         GLA_REQ_V(0, rv0); GLA_REQ_V(1, rv1); GLA_REQ_V(2, rv2); GLA_REQ_V(3, rv3);                  \
     } while (0)
     // two 16-bit halves of a word are rows d and d + 1
@@ -204,8 +215,10 @@ __global__ __launch_bounds__(GLA_WALK_THREADS) void gla_walk_kernel(
         const int p0 = base + place(d), p1 = base + place((d) + 1);                                  \
         q_s[p0] = __uint_as_float((word_q) << 16) * q_scale;                                         \
         q_s[p1] = __uint_as_float((word_q) & 0xffff0000u) * q_scale;                                 \
-        k_s[p0] = __uint_as_float((word_k) << 16);                                                   \
-        k_s[p1] = __uint_as_float((word_k) & 0xffff0000u);                                           \
+        if constexpr (!KF) {                                                                         \
+            k_s[p0] = __uint_as_float((word_k) << 16);                                               \
+            k_s[p1] = __uint_as_float((word_k) & 0xffff0000u);                                       \
+        }                                                                                            \
     } while (0)
 #define GLA_DEP_QK(i, Q, K)                                                                          \
     do {                                                                                             \
@@ -218,11 +231,12 @@ __global__ __launch_bounds__(GLA_WALK_THREADS) void gla_walk_kernel(
             GLA_PUT(Q.w, K.w, d0 + 6);                                                               \
         }                                                                                            \
     } while (0)
-#define GLA_DEP_A(i, A)                                                                              \
+#define GLA_DEP_F(i, A, DST)                                                                         \
     do {   /* four rows of one lane (ROWS is a multiple of 4) */                                     \
         const int idx = tid + (i) * threads;                                                         \
-        if (idx < dnt * d4) *reinterpret_cast<float4*>(al_s + (idx / d4) * Dp + place((idx % d4) * 4)) = A; \
+        if (idx < dnt * d4) *reinterpret_cast<float4*>(DST + (idx / d4) * Dp + place((idx % d4) * 4)) = A; \
     } while (0)
+#define GLA_DEP_A(i, A) GLA_DEP_F(i, A, al_s)
 #define GLA_DEP_V(i, V)                                                                              \
     do {                                                                                             \
         const int idx = tid + (i) * threads;                                                         \
@@ -234,6 +248,10 @@ __global__ __launch_bounds__(GLA_WALK_THREADS) void gla_walk_kernel(
         GLA_DEP_QK(0, rq0, rk0); GLA_DEP_QK(1, rq1, rk1); GLA_DEP_QK(2, rq2, rk2); GLA_DEP_QK(3, rq3, rk3); \
         GLA_DEP_A(0, ra0); GLA_DEP_A(1, ra1); GLA_DEP_A(2, ra2); GLA_DEP_A(3, ra3);                  \
         GLA_DEP_A(4, ra4); GLA_DEP_A(5, ra5); GLA_DEP_A(6, ra6); GLA_DEP_A(7, ra7);                  \
+        if constexpr (KF) {                                                                          \
+            GLA_DEP_F(0, rf0, k_s); GLA_DEP_F(1, rf1, k_s); GLA_DEP_F(2, rf2, k_s); GLA_DEP_F(3, rf3, k_s); \
+            GLA_DEP_F(4, rf4, k_s); GLA_DEP_F(5, rf5, k_s); GLA_DEP_F(6, rf6, k_s); GLA_DEP_F(7, rf7, k_s); \
+        }                                                                                            \
         GLA_DEP_V(0, rv0); GLA_DEP_V(1, rv1); GLA_DEP_V(2, rv2); GLA_DEP_V(3, rv3);                  \
     } while (0)
     // One round before the first block only requests it (each of the two steps is written once, so that the pieces
@@ -299,6 +317,8 @@ __global__ __launch_bounds__(GLA_WALK_THREADS) void gla_walk_kernel(
 
 #undef GLA_REQ_QK
 #undef GLA_REQ_A
+#undef GLA_REQ_F
+#undef GLA_DEP_F
 #undef GLA_REQ_V
 #undef GLA_REQUEST
 #undef GLA_PUT
@@ -415,21 +435,28 @@ static int launch_recurrence(const void* proj, int row_stride, int q_col, int k_
     const int w_rows = (D + 15) / 16;
     const int w_rows_t = w_rows <= 4 ? 4 : w_rows <= 8 ? 8 : w_rows <= 16 ? 16 : 32;
     const size_t w_lds = (size_t)GLA_WALK_TOKENS * (3 * 16 * w_rows_t + 2 * w_slice) * sizeof(float);
-    const bool ahead = prompt && dtype == SIA_BF16 && !k_f32 && q_share == 1 &&
-                       state_stride == (long long)n_heads * D * Dv && D % 8 == 0 && row_stride % 8 == 0 &&
-                       q_col % 8 == 0 && k_col % 8 == 0 && ((uintptr_t)proj % 16) == 0 &&
+    const bool ahead = prompt && dtype == SIA_BF16 && D % 8 == 0 && row_stride % 8 == 0 && q_col % 8 == 0 &&
+                       (k_f32 ? ((uintptr_t)k_f32 % 16) == 0 : k_col % 8 == 0) && ((uintptr_t)alpha % 16) == 0 &&
+                       ((uintptr_t)proj % 16) == 0 &&
                        GLA_WALK_TOKENS * (D / 8) <= 4 * GLA_WALK_THREADS && w_lds <= 60 * 1024 && w_rows_t <= 16;
     float* raw = (sliced || ahead || want_raw) ? raw_space : nullptr;
     if (raw_used) *raw_used = raw != nullptr;
     if (ahead) {
         dim3 wgrid(n_seqs, n_heads, (Dv + w_slice - 1) / w_slice), wblock(GLA_WALK_THREADS);
+#define WALK_AS(ROWS, COLS, KF)                                                                                      \
+    hipLaunchKernelGGL((gla_walk_kernel<ROWS, COLS, KF>), wgrid, wblock, w_lds, stream, (const bf16_t*)proj,         \
+                       row_stride, q_col, k_col, v_col, alpha, k_f32, q_share, state, state_stride, cu_q, slots,     \
+                       n_heads, D, Dv, q_scale, raw)
 #define WALK(ROWS, COLS)                                                                                             \
-    hipLaunchKernelGGL((gla_walk_kernel<ROWS, COLS>), wgrid, wblock, w_lds, stream, (const bf16_t*)proj, row_stride, \
-                       q_col, k_col, v_col, alpha, state, cu_q, slots, n_heads, D, Dv, q_scale, raw)
+    do {                                                                                                             \
+        if (k_f32) WALK_AS(ROWS, COLS, true);                                                                        \
+        else WALK_AS(ROWS, COLS, false);                                                                             \
+    } while (0)
         if (w_rows_t == 4) WALK(4, 2);
         else if (w_rows_t == 8) WALK(8, 2);
         else WALK(16, 2);
 #undef WALK
+#undef WALK_AS
     } else {
 #define LAUNCH(T, ROWS)                                                                                              \
     hipLaunchKernelGGL((gla_recurrent_kernel<T, ROWS>), grid, block, bytes(TB), stream, (const T*)proj, row_stride,  \

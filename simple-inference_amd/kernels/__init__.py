@@ -111,6 +111,8 @@ _ATTN_SIGNATURES = {
                          _c_ptr],
     "sia_attn_decode_ex": [_c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
                            _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int, _c_ptr, _c_int, _c_ptr],
+    "sia_attn_decode_shared": [_c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
+                               _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int, _c_ptr, _c_int, _c_ptr],
     "sia_attn_prefill_ex": [_c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr,
                             _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float,
                             _c_int, _c_int, _c_ptr, _c_ptr],
@@ -1220,8 +1222,12 @@ class HipKernels:
         span = min(b for b in (window, chunk) if b > 0) if (window > 0 or chunk > 0) else 0   # most keys a query sees
         if plans is not None and key in plans:
             return plans[key]
+        # the decode kernel takes up to 16 query heads a key/value head (and what its LDS holds of their states): more
+        # are dealt out as several groups that read the same head
         group = n_heads // n_kv_heads
-        n_dec = ctx.n_decode_seqs if group <= 16 and 4 * group * (head_dim + 2) * 4 <= 65536 else 0
+        share = next(s for s in range(1, group + 1)
+                     if group % s == 0 and group // s <= 16 and 4 * (group // s) * (head_dim + 2) * 4 <= 65536)
+        n_dec = ctx.n_decode_seqs
         max_splits, ws_acc, ws_ml = 1, None, None
         if n_dec:
             # How many workgroups share a (sequence, kv head) is the kernel's decision, from that sequence's own
@@ -1229,7 +1235,7 @@ class HipKernels:
             max_splits = lib.sia_attn_decode_max_splits(int(ctx.kv_bound or ctx.max_kv_len), span)
             ws_acc, ws_ml = (
                 torch.empty((floats,), dtype=torch.float32, device=device) if floats else None
-                for floats in (lib.sia_attn_decode_workspace(n_dec, n_heads, n_kv_heads, max_splits, which)
+                for floats in (lib.sia_attn_decode_workspace(n_dec, n_heads, n_kv_heads * share, max_splits, which)
                                for which in (0, 1)))
         tiles = (0, 0, 0, 0, 0)
         if n_dec < ctx.n_seqs:
@@ -1239,7 +1245,7 @@ class HipKernels:
                           for rows in (lib.sia_attn_prefill_rows(), lib.sia_attn_prefill_rows_split(),
                                        lib.sia_attn_prefill_rows_long()))
             tiles += (int(max(ctx.q_lens[n_dec:])), int(getattr(ctx, "max_run_kv_len", 0) or ctx.max_kv_len))
-        plan = (n_dec, max_splits, ws_acc, ws_ml, tiles)
+        plan = (n_dec, max_splits, ws_acc, ws_ml, tiles, share)
         if plans is None:
             try:
                 ctx.attention_plans = plans = {}
@@ -1252,14 +1258,14 @@ class HipKernels:
         lib = self._attn_lib(head_dim)
         width = qkv.shape[1]
         table = cache.block_table
-        n_dec, max_splits, ws_acc, ws_ml, (n_tiles, n_tiles_split, n_tiles_long, q_bound, kv_bound) = \
+        n_dec, max_splits, ws_acc, ws_ml, (n_tiles, n_tiles_split, n_tiles_long, q_bound, kv_bound), share = \
             self._attention_plan(lib, qkv.device, n_heads, n_kv_heads, head_dim, window, ctx, chunk)
         if n_dec:
-            self._check(lib.sia_attn_decode_ex(
+            self._check(lib.sia_attn_decode_shared(
                 _ptr(qkv), width, _ptr(cache.k_pages), _ptr(cache.v_pages), _ptr(table), table.shape[1],
                 _ptr(ctx.cu_q), _ptr(ctx.kv_len), _ptr(out), _ptr(ws_acc), _ptr(ws_ml), n_dec, n_heads,
-                n_kv_heads, cache.page_size, float(scale), window, chunk, _ptr(sinks), max_splits, self._stream()),
-                "attn_decode")
+                n_kv_heads * share, share, cache.page_size, float(scale), window, chunk, _ptr(sinks), max_splits,
+                self._stream()), "attn_decode")
         if n_dec < ctx.n_seqs:
             self._check(lib.sia_attn_prefill_ex(
                 _ptr(qkv), width, _ptr(cache.k_pages), _ptr(cache.v_pages), _ptr(table), table.shape[1],
@@ -1331,8 +1337,10 @@ class HipKernels:
         if not all(self._library_can(M, n, k) for n, k in ((width, H), (H, Q), (2 * I, H), (H, I))):
             return None
         lib = self._attn_lib(own.head_dim)
-        n_dec, max_splits, ws_acc, ws_ml, tiles = self._attention_plan(lib, device, own.n_heads, own.n_kv, own.head_dim,
-                                                                       own.window, ctx)
+        n_dec, max_splits, ws_acc, ws_ml, tiles, share = self._attention_plan(lib, device, own.n_heads, own.n_kv,
+                                                                              own.head_dim, own.window, ctx)
+        if share != 1:      # the library's step calls the decode kernel with the heads' own grouping
+            return None
         new = lambda n: torch.empty((M, n), dtype=torch.bfloat16, device=device)
         buffers = [new(H), new(width), new(Q), new(H), new(2 * I), new(I), new(H)]
         fn = lambda f: ctypes.cast(f, ctypes.c_void_p).value

@@ -433,11 +433,14 @@ LATENTS = [
         factor=16.0, original=128, fast=32.0, slow=1.0)}),
     dict(heads=5, dim=12, rot_dim=6, vdim=20, q_rank=14, kv_rank=22, scale=0.4, rot={"base": 777.0, "dims": 4}),
     dict(heads=2, dim=128, rot_dim=64, vdim=128, q_rank=96, kv_rank=192, scale=0.07, rot={"base": 10000.0, "dims": 64}),
+    # more heads on the one cached row than a decode workgroup takes: dealt out as two groups of 12, as 17 of one
+    dict(heads=24, dim=16, rot_dim=16, vdim=16, q_rank=32, kv_rank=48, scale=0.15, rot={"base": 10000.0, "dims": 16}),
+    dict(heads=17, dim=8, rot_dim=8, vdim=24, q_rank=24, kv_rank=24, scale=0.2, rot={"base": 500.0, "dims": 8}),
 ]
 
 
 @pytest.mark.parametrize("backend", BACKENDS)
-@pytest.mark.parametrize("m,page", list(zip(LATENTS, [8, 16, 16, 4, 16])))
+@pytest.mark.parametrize("m,page", list(zip(LATENTS, [8, 16, 16, 4, 16, 16, 8])))
 def test_latent_attention_in_prompts_portions_and_decoding_and_from_another_layers_pages(backend, m, page):
     k, dev, dtype, tol = setup(backend)
     g = torch.Generator().manual_seed(m["kv_rank"])
