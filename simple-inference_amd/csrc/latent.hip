@@ -91,6 +91,33 @@ SIA_EXPORT int sia_latent_prepare(const void* proj, int row_stride, int q_rank, 
     return SIA_LAUNCH_CHECK();
 }
 
+// Behind a head's outputs: the head's tail, its first rotary_dim elements turned in neighbouring pairs, and zeros up to
+// the head's stride, for tokens n0 .. n0 + tokens - 1 of head h, by all threads of the workgroup.
+template <typename T>
+__device__ __forceinline__ void headwise_tail(const T* __restrict__ x, int x_row, int in_stride, T* __restrict__ y,
+                                              int y_row, int out_stride, int n_tokens, int in_dim, int out_dim, int tail,
+                                              int rotary_dim, const float* __restrict__ cos_t,
+                                              const float* __restrict__ sin_t, const int* __restrict__ positions,
+                                              int n0, int tokens, int h) {
+    const int rest = out_stride - out_dim, half = rotary_dim / 2;
+    for (int idx = threadIdx.x; idx < tokens * rest; idx += blockDim.x) {
+        const int n = n0 + idx / rest, i = idx % rest;
+        if (n >= n_tokens) break;
+        float v = 0.f;
+        if (i < tail) {
+            const T* src = x + (size_t)n * x_row + (size_t)h * in_stride + in_dim;
+            v = to_float(src[i]);
+            if (i < rotary_dim) {
+                const int pos = positions[n];
+                const float other = to_float(src[i ^ 1]);
+                const float c = cos_t[(size_t)pos * half + i / 2], s = sin_t[(size_t)pos * half + i / 2];
+                v = (i & 1) ? v * c + other * s : v * c - other * s;
+            }
+        }
+        y[(size_t)n * y_row + (size_t)h * out_stride + out_dim + i] = from_float<T>(v);
+    }
+}
+
 #define HW_TOKENS 16
 #define HW_OUTS 64
 #define HW_K 32
@@ -133,24 +160,98 @@ __global__ __launch_bounds__(256) void headwise_linear_kernel(const T* __restric
         if (n < n_tokens && o0 + o < out_dim) y[(size_t)n * y_row + (size_t)h * out_stride + o0 + o] = from_float<T>(acc[t]);
     }
     if (blockIdx.z != 0) return;
-    // behind the outputs: the head's tail, turned, and zeros up to the head's stride
-    const int rest = out_stride - out_dim, half = rotary_dim / 2;
-    for (int idx = tid; idx < HW_TOKENS * rest; idx += blockDim.x) {
-        const int n = n0 + idx / rest, i = idx % rest;
-        if (n >= n_tokens) break;
-        float v = 0.f;
-        if (i < tail) {
-            const T* src = x + (size_t)n * x_row + (size_t)h * in_stride + in_dim;
-            v = to_float(src[i]);
-            if (i < rotary_dim) {
-                const int pos = positions[n];
-                const float other = to_float(src[i ^ 1]);
-                const float c = cos_t[(size_t)pos * half + i / 2], s = sin_t[(size_t)pos * half + i / 2];
-                v = (i & 1) ? v * c + other * s : v * c - other * s;
-            }
+    headwise_tail<T>(x, x_row, in_stride, y, y_row, out_stride, n_tokens, in_dim, out_dim, tail, rotary_dim, cos_t, sin_t,
+                     positions, n0, HW_TOKENS, h);
+}
+
+// A step of few rows (decode): a wave an output element of a head, for all the rows; the head's weight row is read once
+// from memory (again from the cache for every further row), sums in float.
+template <typename T>
+__global__ __launch_bounds__(256) void headwise_rows_kernel(const T* __restrict__ x, int x_row, int in_stride,
+                                                            const T* __restrict__ w, T* __restrict__ y, int y_row,
+                                                            int out_stride, int n_tokens, int in_dim, int out_dim,
+                                                            int tail, int rotary_dim, const float* __restrict__ cos_t,
+                                                            const float* __restrict__ sin_t,
+                                                            const int* __restrict__ positions) {
+    const int h = blockIdx.y, wave = threadIdx.x / SIA_WAVE, lane = threadIdx.x % SIA_WAVE;
+    const int o = blockIdx.x * (blockDim.x / SIA_WAVE) + wave;
+    if (o < out_dim) {
+        const T* wr = w + ((size_t)h * out_dim + o) * in_dim;
+        for (int n = 0; n < n_tokens; ++n) {
+            const T* xr = x + (size_t)n * x_row + (size_t)h * in_stride;
+            float acc = 0.f;
+            for (int k = lane; k < in_dim; k += SIA_WAVE) acc += to_float(wr[k]) * to_float(xr[k]);
+            acc = wave_sum(acc);
+            if (lane == 0) y[(size_t)n * y_row + (size_t)h * out_stride + o] = from_float<T>(acc);
         }
-        y[(size_t)n * y_row + (size_t)h * out_stride + out_dim + i] = from_float<T>(v);
     }
+    if (blockIdx.x != 0) return;
+    headwise_tail<T>(x, x_row, in_stride, y, y_row, out_stride, n_tokens, in_dim, out_dim, tail, rotary_dim, cos_t, sin_t,
+                     positions, 0, n_tokens, h);
+}
+
+// Many rows in bfloat16 (prompts): matrix cores.  A workgroup 128 tokens and 32 output columns of a head, a wave 32 of
+// the tokens: v_mfma_f32_16x16x32_bf16 with the weights' rows as first operand and the tokens' rows as second, both read
+// k-contiguous from memory in 16-byte pieces (in_dim, the strides and the rows' starts multiples of 8 elements); what
+// lies beyond in_dim in the last step of 32 is zero.
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 hw_bf16x8;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float hw_floatx4;
+
+__global__ __launch_bounds__(256) void headwise_mfma_kernel(const bf16_t* __restrict__ x, int x_row, int in_stride,
+                                                            const bf16_t* __restrict__ w, bf16_t* __restrict__ y,
+                                                            int y_row, int out_stride, int n_tokens, int in_dim,
+                                                            int out_dim, int tail, int rotary_dim,
+                                                            const float* __restrict__ cos_t,
+                                                            const float* __restrict__ sin_t,
+                                                            const int* __restrict__ positions) {
+    const int h = blockIdx.y, o0 = blockIdx.z * 32, n0 = blockIdx.x * 128;
+    const int wave = threadIdx.x / SIA_WAVE, lane = threadIdx.x % SIA_WAVE, r = lane & 15, g = lane >> 4;
+    const int t0 = n0 + wave * 32;
+    if (t0 < n_tokens) {
+        const bf16_t* xp[2];
+        const bf16_t* wp[2];
+#pragma unroll
+        for (int mb = 0; mb < 2; ++mb)
+            xp[mb] = x + (size_t)min(t0 + mb * 16 + r, n_tokens - 1) * x_row + (size_t)h * in_stride + g * 8;
+#pragma unroll
+        for (int nb = 0; nb < 2; ++nb)
+            wp[nb] = w + ((size_t)h * out_dim + min(o0 + nb * 16 + r, out_dim - 1)) * in_dim + g * 8;
+        hw_floatx4 acc[2][2];
+#pragma unroll
+        for (int nb = 0; nb < 2; ++nb)
+#pragma unroll
+            for (int mb = 0; mb < 2; ++mb) acc[nb][mb] = hw_floatx4{0.f, 0.f, 0.f, 0.f};
+        const hw_bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+        for (int k = 0; k < in_dim; k += 32) {
+            const bool live = k + g * 8 < in_dim;
+            hw_bf16x8 a[2], b[2];
+#pragma unroll
+            for (int mb = 0; mb < 2; ++mb) b[mb] = live ? *reinterpret_cast<const hw_bf16x8*>(xp[mb] + k) : zero;
+#pragma unroll
+            for (int nb = 0; nb < 2; ++nb) a[nb] = live ? *reinterpret_cast<const hw_bf16x8*>(wp[nb] + k) : zero;
+#pragma unroll
+            for (int nb = 0; nb < 2; ++nb)
+#pragma unroll
+                for (int mb = 0; mb < 2; ++mb)
+                    acc[nb][mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[nb], b[mb], acc[nb][mb], 0, 0, 0);
+        }
+        // acc[nb][mb][i]: output column o0 + nb * 16 + 4g + i of token t0 + mb * 16 + r
+#pragma unroll
+        for (int mb = 0; mb < 2; ++mb) {
+            const int n = t0 + mb * 16 + r;
+            if (n >= n_tokens) continue;
+#pragma unroll
+            for (int nb = 0; nb < 2; ++nb)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int c = o0 + nb * 16 + 4 * g + i;
+                    if (c < out_dim) y[(size_t)n * y_row + (size_t)h * out_stride + c] = float_to_bf16(acc[nb][mb][i]);
+                }
+        }
+    }
+    if (blockIdx.z != 0) return;
+    headwise_tail<bf16_t>(x, x_row, in_stride, y, y_row, out_stride, n_tokens, in_dim, out_dim, tail, rotary_dim, cos_t,
+                          sin_t, positions, n0, 128, h);
 }
 
 SIA_EXPORT int sia_headwise_linear(const void* x, int x_row, int in_stride, const void* w, void* y, int y_row,
@@ -164,6 +265,28 @@ SIA_EXPORT int sia_headwise_linear(const void* x, int x_row, int in_stride, cons
         (out_dim + HW_OUTS - 1) / HW_OUTS > 65535)
         return SIA_BAD_ARGUMENT;
     dim3 grid((n_tokens + HW_TOKENS - 1) / HW_TOKENS, n_heads, (out_dim + HW_OUTS - 1) / HW_OUTS), block(256);
+    if (n_tokens <= 16 && (out_dim + 3) / 4 <= 65535) {
+        dim3 rgrid((out_dim + 3) / 4, n_heads);
+        if (dtype == SIA_F32)
+            hipLaunchKernelGGL(headwise_rows_kernel<float>, rgrid, block, 0, stream, (const float*)x, x_row, in_stride,
+                               (const float*)w, (float*)y, y_row, out_stride, n_tokens, in_dim, out_dim, tail,
+                               rotary_dim, cos_t, sin_t, positions);
+        else if (dtype == SIA_BF16)
+            hipLaunchKernelGGL(headwise_rows_kernel<bf16_t>, rgrid, block, 0, stream, (const bf16_t*)x, x_row, in_stride,
+                               (const bf16_t*)w, (bf16_t*)y, y_row, out_stride, n_tokens, in_dim, out_dim, tail,
+                               rotary_dim, cos_t, sin_t, positions);
+        else
+            return SIA_BAD_ARGUMENT;
+        return SIA_LAUNCH_CHECK();
+    }
+    if (dtype == SIA_BF16 && in_dim % 8 == 0 && x_row % 8 == 0 && in_stride % 8 == 0 && ((uintptr_t)x % 16) == 0 &&
+        ((uintptr_t)w % 16) == 0 && (out_dim + 31) / 32 <= 65535) {
+        dim3 mgrid((n_tokens + 127) / 128, n_heads, (out_dim + 31) / 32);
+        hipLaunchKernelGGL(headwise_mfma_kernel, mgrid, block, 0, stream, (const bf16_t*)x, x_row, in_stride,
+                           (const bf16_t*)w, (bf16_t*)y, y_row, out_stride, n_tokens, in_dim, out_dim, tail, rotary_dim,
+                           cos_t, sin_t, positions);
+        return SIA_LAUNCH_CHECK();
+    }
     if (dtype == SIA_F32)
         hipLaunchKernelGGL(headwise_linear_kernel<float>, grid, block, 0, stream, (const float*)x, x_row, in_stride,
                            (const float*)w, (float*)y, y_row, out_stride, n_tokens, in_dim, out_dim, tail, rotary_dim,

@@ -530,3 +530,28 @@ def test_one_far_latent_is_found_among_hundreds_and_one_ahead_is_not(backend, de
         v = (kv[0][place] @ T64["p.uv"].T) @ T64["p.o"].T
         seen = place <= ask
         assert (float((got - v).abs().max()) < 0.05 * float(v.abs().max())) == seen, (place, decoding)
+
+
+@pytest.mark.parametrize("backend", BACKENDS)
+@pytest.mark.parametrize("heads,in_dim,out_dim,tail,rotary,spare", [(3, 16, 40, 8, 8, 0), (24, 128, 192, 64, 64, 0), (5, 12, 22, 6, 4, 4),
+                                                                    (2, 192, 128, 0, 0, 64), (1, 24, 24, 16, 8, 8), (4, 40, 100, 0, 0, 0)])
+@pytest.mark.parametrize("n", [1, 7, 16, 45, 300])
+def test_a_product_per_head_with_the_turned_tail_behind_it(backend, heads, in_dim, out_dim, tail, rotary, spare, n):
+    """Few rows, many rows, sizes the wide loads take and sizes they do not: the same numbers."""
+    k, dev, dtype, tol = setup(backend)
+    g = torch.Generator().manual_seed(heads * in_dim + n)
+    in_stride, out_stride = in_dim + tail + spare, out_dim + tail + 3
+    x, x64 = lowered(rnd(g, n, heads * in_stride), dtype, dev)
+    w, w64 = lowered(rnd(g, heads, out_dim, in_dim, std=in_dim ** -0.5), dtype, dev)
+    positions = torch.randint(0, 500, (n,), generator=g)
+    cos64, sin64 = plain.rotary_tables(500, {"dims": max(rotary, 2), "base": 1000.0})
+    rotation = (rotary, f32(cos64, dev), f32(sin64, dev), positions.to(torch.int32).to(dev)) if rotary else None
+    got = k.headwise_linear(x, w, in_stride, out_stride, tail=tail, rotation=rotation).double().cpu().view(n, heads, out_stride)
+    xs = x64.view(n, heads, in_stride)
+    close(got[:, :, :out_dim], torch.einsum("nhi,hoi->nho", xs[:, :, :in_dim], w64), tol)
+    if tail:
+        behind = xs[:, :, in_dim:in_dim + tail]
+        if rotary:
+            behind = plain.rotate_pairs(behind, rounded(cos64)[positions], rounded(sin64)[positions])
+        close(got[:, :, out_dim:out_dim + tail], behind, tol)
+    assert float(got[:, :, out_dim + tail:].abs().max()) == 0
