@@ -25,6 +25,17 @@ def _feduzen_layer(ff, weights_of=None):
     return layer
 
 
+_FAMEPEL_LATENT = {"type": "latent_attention",
+                   "mixer": {"dim": 64, "heads": 8, "kv_rank": 96, "q_rank": 192, "rot_dim": 32, "vdim": 64, "scale": 0.1,
+                             "rot": {"base": 10000.0, "dims": 32,
+                                     "scaling": {"factor": 4.0, "original": 2048, "fast": 32.0, "slow": 1.0}}}}
+
+
+def _famepel_layer(mixer):
+    return dict(mixer, mlp={"kind": "moe", "expert": {"ff": 256},
+                            "router": {"experts": 8, "top": 2, "scale": 2.0, "groups": {"count": 4, "keep": 2}}})
+
+
 def _mogisun_layer(kind, moe):
     if kind == "attention":
         mixer = {"heads": 8, "kv_heads": 2, "dim": 64, "vdim": 64, "scale": 0.125, "q_temp": {"coef": 0.2, "every": 512}}
@@ -75,6 +86,18 @@ PRESETS = {
         "logit_softcap": 30.0, "loop": {"start": 1, "stop": 5, "times": 2},
         "layers": [_mogisun_layer("attention", False), _mogisun_layer("gla", True), _mogisun_layer("attention", False),
                    _mogisun_layer("gla", True), _mogisun_layer("attention", False), _mogisun_layer("gla", True)],
+    },
+    # a small model of the Famepel design: its three mixers in turn, the last layer reading the third's latent, grouped
+    # experts
+    "famepel-small": {
+        "architecture": "Famepel", "vocab": 4096, "width": 512, "norm": {"eps": 1e-6}, "embedding": {"scale": 8.0},
+        "layers": [_famepel_layer({"type": "mamba2", "mixer": {"conv": 4, "groups": 2, "heads": 8, "norm_groups": 2,
+                                                                 "state": 64, "vdim": 64}}),
+                   _famepel_layer({"type": "hgrn2", "mixer": {"dim": 64, "heads": 8, "vdim": 64}}),
+                   _famepel_layer(_FAMEPEL_LATENT),
+                   _famepel_layer({"type": "mamba2", "mixer": {"conv": 4, "groups": 2, "heads": 8, "norm_groups": 2,
+                                                                 "state": 64, "vdim": 64}}),
+                   _famepel_layer(dict(_FAMEPEL_LATENT, mixer=dict(_FAMEPEL_LATENT["mixer"], kv_from=2)))],
     },
     "tiny-a": {
         "architectures": ["LlamaForCausalLM"], "model_type": "llama",

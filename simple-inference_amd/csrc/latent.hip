@@ -13,6 +13,8 @@
 // headwise_linear: y[n, h, o] = sum_i x[n, h, i] * w[h, o, i] for every head, x rows in_stride apart per head, y rows
 // out_stride apart; a head's ``tail`` elements behind the in_dim inputs are copied behind the out_dim outputs, with
 // their first rotary_dim elements turned as above, and the rest of a head's out_stride is set to zero.  Float sums.
+// Three forms: a wave an output element for steps of up to 16 rows, matrix cores for more rows in bfloat16 where the
+// 16-byte loads are aligned, and an LDS-tiled form on the vector units for everything else (float32, odd sizes).
 #include "common.h"
 
 template <typename T>
