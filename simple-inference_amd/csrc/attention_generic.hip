@@ -18,7 +18,8 @@
 // (reference: kernels/attention_kernel.py:184-251, :516-586).  Everything is float.
 #include "common.h"
 
-#define ATTN_MAX_HEAD_DIM 256
+#define ATTN_MAX_HEAD_DIM 640        // of this kernel: wide enough for a cached latent row of 512 + 128
+#define ATTN_MAX_WRITTEN_HEAD_DIM 256  // of the kernels that write rotated keys and values per head into the pages
 
 template <typename T>
 __global__ __launch_bounds__(SIA_WAVE) void attention_generic_kernel(
@@ -43,7 +44,7 @@ __global__ __launch_bounds__(SIA_WAVE) void attention_generic_kernel(
     __syncthreads();
 
     float m = -INFINITY, l = 0.f;
-    float acc[ATTN_MAX_HEAD_DIM / SIA_WAVE] = {0.f, 0.f, 0.f, 0.f};
+    float acc[ATTN_MAX_HEAD_DIM / SIA_WAVE] = {};
 
     for (int c0 = (lo / SIA_WAVE) * SIA_WAVE; c0 <= pos; c0 += SIA_WAVE) {
         const int j = c0 + lane;
@@ -93,8 +94,10 @@ __global__ __launch_bounds__(SIA_WAVE) void attention_generic_kernel(
     }
 }
 
-// The largest head size any attention kernel of this package takes (a model is checked against it when it is built).
-SIA_EXPORT int sia_attention_max_head_dim() { return ATTN_MAX_HEAD_DIM; }
+// The largest head size the kernels of a mixer with keys and values per head take (a model is checked against it when
+// it is built), and the largest row this kernel reads from pages that somebody else wrote.
+SIA_EXPORT int sia_attention_max_head_dim() { return ATTN_MAX_WRITTEN_HEAD_DIM; }
+SIA_EXPORT int sia_attention_generic_max_head_dim() { return ATTN_MAX_HEAD_DIM; }
 
 SIA_EXPORT int sia_attention_generic(const void* q, int q_row_stride, const void* k_pages, const void* v_pages,
                                      const int* block_table, int table_width, const int* seq_of_token,

@@ -80,6 +80,7 @@ _SIGNATURES = {
                               _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int, _c_ptr, _c_int,
                               _c_ptr],
     "sia_attention_max_head_dim": [],
+    "sia_attention_generic_max_head_dim": [],
     "sia_gemm_generic": [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr],
     "sia_prenorm_block": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_int, _c_ptr],
     "sia_sample": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr],
@@ -1171,10 +1172,11 @@ class HipKernels:
                               f"{ctx.max_kv_len} positions with pages of {page_size}")
 
     # -- attention ---------------------------------------------------------------
-    def check_attention_geometry(self, n_heads: int, n_kv_heads: int, head_dim: int) -> None:
+    def check_attention_geometry(self, n_heads: int, n_kv_heads: int, head_dim: int, own_writer: bool = False) -> None:
         """Raises for head counts and sizes that no attention kernel here takes.  A mixer calls it when the model is
-        built, so that such a model is refused before it is loaded, not at its first step."""
-        limit = self.core.sia_attention_max_head_dim()
+        built, so that such a model is refused before it is loaded, not at its first step.  ``own_writer``: the mixer
+        fills the pages with a kernel of its own that has no limit, so the page attention's limit is the only one."""
+        limit = self.core.sia_attention_generic_max_head_dim() if own_writer else self.core.sia_attention_max_head_dim()
         if not 0 < head_dim <= limit:
             raise KernelError(f"head size {head_dim} is outside what the attention kernels take (1 to {limit})")
         if n_kv_heads <= 0 or n_heads <= 0 or n_heads % n_kv_heads:

@@ -56,7 +56,7 @@ class LatentAttention:
         self.key_dim = self.kv_rank + self.rot_dim     # a cached key row: the latent and the shared rotated part
         check = getattr(env.kernels, "check_attention_geometry", None)
         if check is not None:
-            check(self.num_heads, 1, self.key_dim)
+            check(self.num_heads, 1, self.key_dim, own_writer=True)
         page_dim = getattr(env.kernels, "attention_page_dim", None)
         self.page_dim = page_dim(self.key_dim, self.kv_rank, env.dtype) if page_dim is not None else None
         self.env = env

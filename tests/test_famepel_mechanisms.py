@@ -436,11 +436,13 @@ LATENTS = [
     # more heads on the one cached row than a decode workgroup takes: dealt out as two groups of 12, as 17 of one
     dict(heads=24, dim=16, rot_dim=16, vdim=16, q_rank=32, kv_rank=48, scale=0.15, rot={"base": 10000.0, "dims": 16}),
     dict(heads=17, dim=8, rot_dim=8, vdim=24, q_rank=24, kv_rank=24, scale=0.2, rot={"base": 500.0, "dims": 8}),
+    # a cached row wider than any head the matrix-core attention is built for
+    dict(heads=2, dim=32, rot_dim=32, vdim=40, q_rank=24, kv_rank=288, scale=0.1, rot={"base": 10000.0, "dims": 32}),
 ]
 
 
 @pytest.mark.parametrize("backend", BACKENDS)
-@pytest.mark.parametrize("m,page", list(zip(LATENTS, [8, 16, 16, 4, 16, 16, 8])))
+@pytest.mark.parametrize("m,page", list(zip(LATENTS, [8, 16, 16, 4, 16, 16, 8, 16])))
 def test_latent_attention_in_prompts_portions_and_decoding_and_from_another_layers_pages(backend, m, page):
     k, dev, dtype, tol = setup(backend)
     g = torch.Generator().manual_seed(m["kv_rank"])
