@@ -32,15 +32,30 @@ template <typename T> __device__ __forceinline__ T from_float(float x);
 template <> __device__ __forceinline__ float from_float<float>(float x) { return x; }
 template <> __device__ __forceinline__ bf16_t from_float<bf16_t>(float x) { return float_to_bf16(x); }
 
-// Activations without a gate, in float:  SIA_RELU2: max(z, 0)^2;  SIA_GELU_TANH: 0.5 z (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3))).
-enum SiaActivation { SIA_RELU2 = 0, SIA_GELU_TANH = 1 };
+// Activations without a gate, in float:  SIA_RELU2: max(z, 0)^2;  SIA_GELU_TANH: 0.5 z (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3)));
+// SIA_GELU: 0.5 z (1 + erf(z / sqrt(2))).
+enum SiaActivation { SIA_RELU2 = 0, SIA_GELU_TANH = 1, SIA_GELU = 2 };
 
 __device__ __forceinline__ float activate(float z, int kind) {
     if (kind == SIA_RELU2) {
         const float r = fmaxf(z, 0.f);
         return r * r;
     }
+    if (kind == SIA_GELU) return 0.5f * z * (1.f + erff(z * 0.70710678118654752f));
     return 0.5f * z * (1.f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+}
+
+// Gated activations of a (gate, up) pair, in float.  SIA_GLU_SILU: silu(g) * u.  SIA_GLU_CLAMPED: with g = min(g, limit)
+// and u = clamp(u, -limit, limit):  g * sigmoid(1.702 g) * (u + 1).
+enum SiaGlu { SIA_GLU_SILU = 0, SIA_GLU_CLAMPED = 1 };
+
+__device__ __forceinline__ float gated_activation(float g, float u, int kind, float limit) {
+    if (kind == SIA_GLU_CLAMPED) {
+        g = fminf(g, limit);
+        u = fminf(fmaxf(u, -limit), limit);
+        return g / (1.f + expf(-1.702f * g)) * (u + 1.f);
+    }
+    return g / (1.f + expf(-g)) * u;
 }
 
 // Eight consecutive elements of a row as one register value: 32 bytes of float or 16 of bfloat16.

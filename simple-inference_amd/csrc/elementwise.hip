@@ -41,29 +41,36 @@ SIA_EXPORT int sia_embed(const int* ids, const void* table, float* out, int n_to
 // rows != nullptr: out[i] comes from row rows[i]; residual is not written.
 // The sum of squares is reduced in a fixed order that depends on the row length only.
 // ---------------------------------------------------------------------------------------
-template <typename T>
+// SCALED: the delta is multiplied by a constant, and a second delta with a constant of its own may join it
+// (x = residual + f1 * delta + f2 * delta2); without a weight only the sum is made.
+template <typename T, bool SCALED>
 __global__ void add_rmsnorm_kernel(float* __restrict__ residual, const T* __restrict__ delta,
                                    const float* __restrict__ weight, T* __restrict__ out,
-                                   const int* __restrict__ rows, int hidden, float eps) {
+                                   const int* __restrict__ rows, int hidden, float eps, float f1,
+                                   const T* __restrict__ delta2, float f2) {
     __shared__ float scratch[16];
     const int i_out = blockIdx.x;
     const int row = rows ? rows[i_out] : i_out;
     float* res = residual + (size_t)row * hidden;
     const T* del = delta ? delta + (size_t)row * hidden : nullptr;
+    const T* del2 = (SCALED && delta2) ? delta2 + (size_t)row * hidden : nullptr;
     T* dst = out + (size_t)i_out * hidden;
 
     float ss = 0.f;
     for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
         float x = res[i];
-        if (del) x += to_float(del[i]);
+        if (del) x += SCALED ? f1 * to_float(del[i]) : to_float(del[i]);
+        if (del2) x += f2 * to_float(del2[i]);
         if (!rows && del) res[i] = x;
         ss += x * x;
     }
+    if (SCALED && !weight) return;   // uniform
     ss = block_sum(ss, scratch);
     const float inv = rsqrtf(ss / (float)hidden + eps);
     for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
         float x = res[i];
-        if (rows && del) x += to_float(del[i]);
+        if (rows && del) x += SCALED ? f1 * to_float(del[i]) : to_float(del[i]);
+        if (rows && del2) x += f2 * to_float(del2[i]);
         dst[i] = from_float<T>(x * inv * weight[i]);
     }
 }
@@ -71,34 +78,42 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ residual, const T* __rest
 // The same for rows that one workgroup holds in registers (hidden % 8 == 0, hidden <= 8 * 1024): each
 // thread takes 8 consecutive elements with 16- and 32-byte accesses, every input is read once and all
 // loads (the gain's included) are issued before the first is used.
-template <typename T>
+template <typename T, bool SCALED>
 __global__ void add_rmsnorm_row_kernel(float* __restrict__ residual, const T* __restrict__ delta,
                                        const float* __restrict__ weight, T* __restrict__ out,
-                                       const int* __restrict__ rows, int hidden, float eps) {
+                                       const int* __restrict__ rows, int hidden, float eps, float f1,
+                                       const T* __restrict__ delta2, float f2) {
     __shared__ float scratch[16];
     const int i_out = blockIdx.x;
     const int row = rows ? rows[i_out] : i_out;
     const int i0 = threadIdx.x * 8;
     const bool live = i0 < hidden;
-    float x[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f}, w[8], d[8];
+    float x[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f}, w[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f}, d[8];
     if (live) {
         Vec8<float> vr, vw;
-        Vec8<T> vd;
+        Vec8<T> vd, vd2;
         vr.load(residual + (size_t)row * hidden + i0);
-        vw.load(weight + i0);
+        if (!SCALED || weight) vw.load(weight + i0);
         if (delta) vd.load(delta + (size_t)row * hidden + i0);
+        if (SCALED && delta2) vd2.load(delta2 + (size_t)row * hidden + i0);
         vr.get(x);
-        vw.get(w);
+        if (!SCALED || weight) vw.get(w);
         if (delta) {
             vd.get(d);
 #pragma unroll
-            for (int i = 0; i < 8; ++i) x[i] += d[i];
+            for (int i = 0; i < 8; ++i) x[i] += SCALED ? f1 * d[i] : d[i];
+            if (SCALED && delta2) {
+                vd2.get(d);
+#pragma unroll
+                for (int i = 0; i < 8; ++i) x[i] += f2 * d[i];
+            }
             if (!rows) {
                 vr.set(x);
                 vr.store(residual + (size_t)row * hidden + i0);
             }
         }
     }
+    if (SCALED && !weight) return;   // uniform: only the sum was asked for
     float ss = 0.f;
 #pragma unroll
     for (int i = 0; i < 8; ++i) ss += x[i] * x[i];
@@ -113,30 +128,49 @@ __global__ void add_rmsnorm_row_kernel(float* __restrict__ residual, const T* __
     }
 }
 
-SIA_EXPORT int sia_add_rmsnorm(float* residual, const void* delta, const float* weight, void* out,
-                               const int* rows, int n_out, int hidden, float eps, int dtype,
-                               hipStream_t stream) {
+template <bool SCALED>
+static int launch_add_rmsnorm(float* residual, const void* delta, float f1, const void* delta2, float f2,
+                              const float* weight, void* out, const int* rows, int n_out, int hidden, float eps,
+                              int dtype, hipStream_t stream) {
     if (n_out <= 0) return 0;
     if (dtype != SIA_F32 && dtype != SIA_BF16) return SIA_BAD_ARGUMENT;
     dim3 grid(n_out);
     if (hidden % 8 == 0 && hidden <= 8 * 1024) {
         dim3 block(((hidden / 8 + SIA_WAVE - 1) / SIA_WAVE) * SIA_WAVE);
         if (dtype == SIA_F32)
-            hipLaunchKernelGGL(add_rmsnorm_row_kernel<float>, grid, block, 0, stream, residual, (const float*)delta,
-                               weight, (float*)out, rows, hidden, eps);
+            hipLaunchKernelGGL((add_rmsnorm_row_kernel<float, SCALED>), grid, block, 0, stream, residual,
+                               (const float*)delta, weight, (float*)out, rows, hidden, eps, f1, (const float*)delta2, f2);
         else
-            hipLaunchKernelGGL(add_rmsnorm_row_kernel<bf16_t>, grid, block, 0, stream, residual,
-                               (const bf16_t*)delta, weight, (bf16_t*)out, rows, hidden, eps);
+            hipLaunchKernelGGL((add_rmsnorm_row_kernel<bf16_t, SCALED>), grid, block, 0, stream, residual,
+                               (const bf16_t*)delta, weight, (bf16_t*)out, rows, hidden, eps, f1, (const bf16_t*)delta2,
+                               f2);
         return SIA_LAUNCH_CHECK();
     }
     dim3 block(hidden >= 2048 ? 512 : 256);
     if (dtype == SIA_F32)
-        hipLaunchKernelGGL(add_rmsnorm_kernel<float>, grid, block, 0, stream, residual, (const float*)delta,
-                           weight, (float*)out, rows, hidden, eps);
+        hipLaunchKernelGGL((add_rmsnorm_kernel<float, SCALED>), grid, block, 0, stream, residual, (const float*)delta,
+                           weight, (float*)out, rows, hidden, eps, f1, (const float*)delta2, f2);
     else
-        hipLaunchKernelGGL(add_rmsnorm_kernel<bf16_t>, grid, block, 0, stream, residual, (const bf16_t*)delta,
-                           weight, (bf16_t*)out, rows, hidden, eps);
+        hipLaunchKernelGGL((add_rmsnorm_kernel<bf16_t, SCALED>), grid, block, 0, stream, residual, (const bf16_t*)delta,
+                           weight, (bf16_t*)out, rows, hidden, eps, f1, (const bf16_t*)delta2, f2);
     return SIA_LAUNCH_CHECK();
+}
+
+SIA_EXPORT int sia_add_rmsnorm(float* residual, const void* delta, const float* weight, void* out,
+                               const int* rows, int n_out, int hidden, float eps, int dtype,
+                               hipStream_t stream) {
+    return launch_add_rmsnorm<false>(residual, delta, 1.f, nullptr, 0.f, weight, out, rows, n_out, hidden, eps, dtype,
+                                     stream);
+}
+
+// x = residual + f1 * delta + f2 * delta2 (delta2 may be absent) and, with a weight, the RMS norm of x; without one
+// only the sum is made (rows must then be absent, so that the residual keeps it).
+SIA_EXPORT int sia_add_rmsnorm_scaled(float* residual, const void* delta, float f1, const void* delta2, float f2,
+                                      const float* weight, void* out, const int* rows, int n_out, int hidden,
+                                      float eps, int dtype, hipStream_t stream) {
+    if (!delta || (!weight && rows) || (weight && !out)) return SIA_BAD_ARGUMENT;
+    return launch_add_rmsnorm<true>(residual, delta, f1, delta2, f2, weight, out, rows, n_out, hidden, eps, dtype,
+                                    stream);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -252,12 +286,63 @@ __global__ void activation_kernel(const T* __restrict__ in, T* __restrict__ out,
 // Eight elements a thread; the last thread takes what is left one by one.
 SIA_EXPORT int sia_activation(const void* in, void* out, long long n, int kind, int dtype, hipStream_t stream) {
     if (n <= 0) return 0;
-    if ((dtype != SIA_F32 && dtype != SIA_BF16) || (kind != SIA_RELU2 && kind != SIA_GELU_TANH)) return SIA_BAD_ARGUMENT;
+    if ((dtype != SIA_F32 && dtype != SIA_BF16) || (kind != SIA_RELU2 && kind != SIA_GELU_TANH && kind != SIA_GELU)) return SIA_BAD_ARGUMENT;
     dim3 block(256), grid((unsigned)(((n + 7) / 8 + 255) / 256));
     if (dtype == SIA_F32)
         hipLaunchKernelGGL(activation_kernel<float>, grid, block, 0, stream, (const float*)in, (float*)out, (size_t)n, kind);
     else
         hipLaunchKernelGGL(activation_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)in, (bf16_t*)out, (size_t)n, kind);
+    return SIA_LAUNCH_CHECK();
+}
+
+// ---------------------------------------------------------------------------------------
+// A gated activation of another kind than SwiGLU over rows [gate (I) | up (I)] (``gated_activation`` of common.h),
+// and the sum of up to two matrices with a constant factor each.
+// ---------------------------------------------------------------------------------------
+template <typename T>
+__global__ void glu_kernel(const T* __restrict__ gu, T* __restrict__ out, int inter, int kind, float limit) {
+    const int n = blockIdx.y;
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= inter) return;
+    const T* row = gu + (size_t)n * 2 * inter;
+    out[(size_t)n * inter + i] = from_float<T>(gated_activation(to_float(row[i]), to_float(row[inter + i]), kind, limit));
+}
+
+SIA_EXPORT int sia_glu(const void* gu, void* out, int n_tokens, int inter, int kind, float limit, int dtype,
+                       hipStream_t stream) {
+    if (n_tokens <= 0) return 0;
+    if (n_tokens > 65535 || inter <= 0 || (dtype != SIA_F32 && dtype != SIA_BF16) ||
+        (kind != SIA_GLU_SILU && kind != SIA_GLU_CLAMPED))
+        return SIA_BAD_ARGUMENT;
+    dim3 block(256), grid((inter + 255) / 256, n_tokens);
+    if (dtype == SIA_F32)
+        hipLaunchKernelGGL(glu_kernel<float>, grid, block, 0, stream, (const float*)gu, (float*)out, inter, kind, limit);
+    else
+        hipLaunchKernelGGL(glu_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)gu, (bf16_t*)out, inter, kind, limit);
+    return SIA_LAUNCH_CHECK();
+}
+
+template <typename T>
+__global__ void scaled_sum_kernel(const T* __restrict__ a, float fa, const T* __restrict__ b, float fb,
+                                  T* __restrict__ out, size_t n) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    float x = fa * to_float(a[i]);
+    if (b) x += fb * to_float(b[i]);
+    out[i] = from_float<T>(x);
+}
+
+SIA_EXPORT int sia_scaled_sum(const void* a, float fa, const void* b, float fb, void* out, long long n, int dtype,
+                              hipStream_t stream) {
+    if (n <= 0) return 0;
+    if (!a || !out || (dtype != SIA_F32 && dtype != SIA_BF16)) return SIA_BAD_ARGUMENT;
+    dim3 block(256), grid((unsigned)((n + 255) / 256));
+    if (dtype == SIA_F32)
+        hipLaunchKernelGGL(scaled_sum_kernel<float>, grid, block, 0, stream, (const float*)a, fa, (const float*)b, fb,
+                           (float*)out, (size_t)n);
+    else
+        hipLaunchKernelGGL(scaled_sum_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)a, fa, (const bf16_t*)b, fb,
+                           (bf16_t*)out, (size_t)n);
     return SIA_LAUNCH_CHECK();
 }
 

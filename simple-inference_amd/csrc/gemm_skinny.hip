@@ -395,7 +395,7 @@ SIA_EXPORT int sia_gemm_skinny(const void* X, const void* W, void* Y, int M, int
 SIA_EXPORT int sia_gemm_skinny_act(const void* X, const void* W, void* Y, int M, int N, int K, int activation,
                                    hipStream_t stream) {
     if (M <= 0 || N <= 0) return 0;
-    if (M > 16 || K % 64 || K <= 0 || (activation != SIA_RELU2 && activation != SIA_GELU_TANH)) return SIA_BAD_ARGUMENT;
+    if (M > 16 || K % 64 || K <= 0 || (activation != SIA_RELU2 && activation != SIA_GELU_TANH && activation != SIA_GELU)) return SIA_BAD_ARGUMENT;
     Epilogue ep{};
     ep.activation = activation;
     launch_skinny<bf16_t, EPI_ACT>((const bf16_t*)X, (const bf16_t*)W, (bf16_t*)Y, M, N, K, ep, stream);

@@ -18,12 +18,14 @@
 // score_mode 0: the softmax over the chosen logits alone.  score_mode 1: scores s = sigmoid(z); with n_groups > 0 the
 // experts form n_groups equal groups of neighbours, a group's score is the sum of its two largest s, and only
 // experts of the keep_groups best groups (ties: the lower group) can be chosen; the weights are the chosen s divided
-// by their sum (+ 1e-20), times weight_scale.
+// by their sum (+ 1e-20), times weight_scale.  score_mode 2: scores s = softmax(z) over all experts; the choice goes by
+// s + correction (a float per expert, if given), the weights are the chosen s divided by their sum (+ 1e-20).
 template <typename T>
 __global__ __launch_bounds__(256) void moe_route_kernel(const T* __restrict__ h, const float* __restrict__ router,
                                                          int* __restrict__ ids, float* __restrict__ weights, int width,
                                                          int n_experts, int top, int score_mode, int n_groups,
-                                                         int keep_groups, float weight_scale) {
+                                                         int keep_groups, float weight_scale,
+                                                         const float* __restrict__ correction) {
     __shared__ float logit_s[MOE_MAX_EXPERTS];
     __shared__ float group_s[MOE_MAX_EXPERTS];
     const int n = blockIdx.x, wave = threadIdx.x / SIA_WAVE, lane = threadIdx.x % SIA_WAVE;
@@ -43,6 +45,21 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const T* __restrict__ h,
     }
     __syncthreads();
     if (wave != 0) return;
+    if (score_mode == 2) {
+        // the scores stay in group_s, what the choice goes by takes the logits' place
+        float top_z = -INFINITY, sum = 0.f;
+        for (int e = lane; e < n_experts; e += SIA_WAVE) top_z = fmaxf(top_z, logit_s[e]);
+        top_z = wave_max(top_z);
+        for (int e = lane; e < n_experts; e += SIA_WAVE) sum += expf(logit_s[e] - top_z);
+        sum = wave_sum(sum);
+        for (int e = lane; e < n_experts; e += SIA_WAVE) {
+            const float sc = expf(logit_s[e] - top_z) / sum;
+            group_s[e] = sc;
+            logit_s[e] = correction ? sc + correction[e] : sc;
+        }
+        __builtin_amdgcn_wave_barrier();
+        __threadfence_block();
+    }
     if (score_mode == 1 && n_groups > 0) {
         // a lane a group at a time: the sum of its two largest scores; then keep_groups rounds of a wave-wide best
         // group, and the experts of every other group leave the choice
@@ -97,7 +114,7 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const T* __restrict__ h,
         }
         if (which >= n_experts) { which = k; best = 0.f; }   // logits that are not numbers order nothing: still an expert that exists
         if (k == 0) first = best;
-        const float p = score_mode == 1 ? best : expf(best - first);
+        const float p = score_mode == 1 ? best : score_mode == 2 ? group_s[which] : expf(best - first);
         total += p;
         if (lane == k) { chosen = p; chosen_id = which; }
         if (lane == 0 && which < n_experts) logit_s[which] = -INFINITY;
@@ -106,29 +123,44 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const T* __restrict__ h,
     }
     if (lane < top) {
         ids[(size_t)n * top + lane] = chosen_id;
-        weights[(size_t)n * top + lane] = score_mode == 1 ? chosen / (total + 1e-20f) * weight_scale : chosen / total;
+        weights[(size_t)n * top + lane] = score_mode == 1 ? chosen / (total + 1e-20f) * weight_scale
+                                          : score_mode == 2 ? chosen / (total + 1e-20f) : chosen / total;
     }
 }
 
-SIA_EXPORT int sia_moe_route_ex(const void* h, const float* router, int* ids, float* weights, int n_tokens, int width,
-                                int n_experts, int top, int dtype, int score_mode, int n_groups, int keep_groups,
-                                float weight_scale, hipStream_t stream) {
+static int route(const void* h, const float* router, int* ids, float* weights, int n_tokens, int width, int n_experts,
+                 int top, int dtype, int score_mode, int n_groups, int keep_groups, float weight_scale,
+                 const float* correction, hipStream_t stream) {
     if (n_tokens <= 0) return 0;
     if (n_experts <= 0 || n_experts > MOE_MAX_EXPERTS || top <= 0 || top > n_experts || top > MOE_MAX_TOP ||
-        (score_mode != 0 && score_mode != 1) || n_groups < 0 ||
+        (score_mode != 0 && score_mode != 1 && score_mode != 2) || n_groups < 0 || (correction && score_mode != 2) ||
         (n_groups > 0 && (score_mode != 1 || n_experts % n_groups || keep_groups <= 0 || keep_groups > n_groups ||
                           top > n_experts / n_groups * keep_groups)))
         return SIA_BAD_ARGUMENT;
     dim3 grid(n_tokens), block(256);
     if (dtype == SIA_F32)
         hipLaunchKernelGGL(moe_route_kernel<float>, grid, block, 0, stream, (const float*)h, router, ids, weights, width,
-                           n_experts, top, score_mode, n_groups, keep_groups, weight_scale);
+                           n_experts, top, score_mode, n_groups, keep_groups, weight_scale, correction);
     else if (dtype == SIA_BF16)
         hipLaunchKernelGGL(moe_route_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)h, router, ids, weights,
-                           width, n_experts, top, score_mode, n_groups, keep_groups, weight_scale);
+                           width, n_experts, top, score_mode, n_groups, keep_groups, weight_scale, correction);
     else
         return SIA_BAD_ARGUMENT;
     return SIA_LAUNCH_CHECK();
+}
+
+SIA_EXPORT int sia_moe_route_ex(const void* h, const float* router, int* ids, float* weights, int n_tokens, int width,
+                                int n_experts, int top, int dtype, int score_mode, int n_groups, int keep_groups,
+                                float weight_scale, hipStream_t stream) {
+    return route(h, router, ids, weights, n_tokens, width, n_experts, top, dtype, score_mode, n_groups, keep_groups,
+                 weight_scale, nullptr, stream);
+}
+
+// scores over all experts (score_mode 2) with the vector that corrects the choice
+SIA_EXPORT int sia_moe_route_corrected(const void* h, const float* router, const float* correction, int* ids,
+                                       float* weights, int n_tokens, int width, int n_experts, int top, int dtype,
+                                       hipStream_t stream) {
+    return route(h, router, ids, weights, n_tokens, width, n_experts, top, dtype, 2, 0, 0, 1.f, correction, stream);
 }
 
 SIA_EXPORT int sia_moe_route(const void* h, const float* router, int* ids, float* weights, int n_tokens, int width,
@@ -163,16 +195,17 @@ __device__ __forceinline__ float wave_dot(const T* __restrict__ a, const T* __re
 template <typename T>
 __global__ __launch_bounds__(MOE_WAVES* SIA_WAVE) void moe_gate_up_kernel(
     const T* __restrict__ h, const T* __restrict__ w1, const int* __restrict__ ids, T* __restrict__ act, int width,
-    int ff, int top, bool vec) {
+    int ff, int top, bool vec, int n_real, int glu, float limit) {
     const int slot = blockIdx.x, wave = threadIdx.x / SIA_WAVE, lane = threadIdx.x % SIA_WAVE;
     const int e = ids[slot];
+    if (e >= n_real) return;     // an expert without tensors: the down kernel hands the token's input on
     const T* x = h + (size_t)(slot / top) * width;
     const T* w = w1 + (size_t)e * 2 * ff * width;
     const int f0 = (blockIdx.y * MOE_WAVES + wave) * MOE_PER_WAVE;
     for (int f = f0; f < min(ff, f0 + MOE_PER_WAVE); ++f) {
         const float g = wave_dot<T>(x, w + (size_t)f * width, width, lane, vec);
         const float u = wave_dot<T>(x, w + (size_t)(ff + f) * width, width, lane, vec);
-        if (lane == 0) act[(size_t)slot * ff + f] = from_float<T>(g / (1.f + expf(-g)) * u);
+        if (lane == 0) act[(size_t)slot * ff + f] = from_float<T>(gated_activation(g, u, glu, limit));
     }
 }
 
@@ -180,13 +213,17 @@ template <typename T>
 __global__ __launch_bounds__(MOE_WAVES* SIA_WAVE) void moe_down_kernel(
     const T* __restrict__ act, const T* __restrict__ w2, const int* __restrict__ ids, const float* __restrict__ weights,
     const T* __restrict__ shared, const T* __restrict__ shared_gate, int shared_gate_stride, T* __restrict__ out,
-    int width, int ff, int top, bool vec) {
+    int width, int ff, int top, bool vec, const T* __restrict__ h, int n_real) {
     const int n = blockIdx.x, wave = threadIdx.x / SIA_WAVE, lane = threadIdx.x % SIA_WAVE;
     const int c0 = (blockIdx.y * MOE_WAVES + wave) * MOE_PER_WAVE;
     for (int c = c0; c < min(width, c0 + MOE_PER_WAVE); ++c) {
         float y = 0.f;
         for (int k = 0; k < top; ++k) {
             const int slot = n * top + k;
+            if (ids[slot] >= n_real) {      // wave-uniform
+                y += weights[slot] * to_float(h[(size_t)n * width + c]);
+                continue;
+            }
             const T* w = w2 + ((size_t)ids[slot] * width + c) * ff;
             y += weights[slot] * wave_dot<T>(act + (size_t)slot * ff, w, ff, lane, vec);
         }
@@ -199,20 +236,53 @@ __global__ __launch_bounds__(MOE_WAVES* SIA_WAVE) void moe_down_kernel(
     }
 }
 
-SIA_EXPORT int sia_moe_gate_up(const void* h, const void* w1, const int* ids, void* act, int n_tokens, int width, int ff,
-                               int top, int dtype, hipStream_t stream) {
+// n_real: ids from there on name experts without tensors, which return their input; glu, limit: the experts' gated
+// activation (``gated_activation`` of common.h).
+SIA_EXPORT int sia_moe_gate_up_ex(const void* h, const void* w1, const int* ids, void* act, int n_tokens, int width,
+                                  int ff, int top, int n_real, int glu, float limit, int dtype, hipStream_t stream) {
     if (n_tokens <= 0) return 0;
-    if (width <= 0 || ff <= 0 || top <= 0 || (long long)n_tokens * top > 0x7fffffffLL) return SIA_BAD_ARGUMENT;
+    if (width <= 0 || ff <= 0 || top <= 0 || (long long)n_tokens * top > 0x7fffffffLL || n_real <= 0 ||
+        (glu != SIA_GLU_SILU && glu != SIA_GLU_CLAMPED))
+        return SIA_BAD_ARGUMENT;
     const int per_block = MOE_WAVES * MOE_PER_WAVE;
     dim3 grid(n_tokens * top, (ff + per_block - 1) / per_block), block(MOE_WAVES * SIA_WAVE);
     if (grid.y > 65535) return SIA_BAD_ARGUMENT;
     const bool vec = width % 8 == 0;
     if (dtype == SIA_F32)
         hipLaunchKernelGGL(moe_gate_up_kernel<float>, grid, block, 0, stream, (const float*)h, (const float*)w1, ids,
-                           (float*)act, width, ff, top, vec);
+                           (float*)act, width, ff, top, vec, n_real, glu, limit);
     else if (dtype == SIA_BF16)
         hipLaunchKernelGGL(moe_gate_up_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)h, (const bf16_t*)w1, ids,
-                           (bf16_t*)act, width, ff, top, vec);
+                           (bf16_t*)act, width, ff, top, vec, n_real, glu, limit);
+    else
+        return SIA_BAD_ARGUMENT;
+    return SIA_LAUNCH_CHECK();
+}
+
+SIA_EXPORT int sia_moe_gate_up(const void* h, const void* w1, const int* ids, void* act, int n_tokens, int width, int ff,
+                               int top, int dtype, hipStream_t stream) {
+    return sia_moe_gate_up_ex(h, w1, ids, act, n_tokens, width, ff, top, 0x7fffffff, SIA_GLU_SILU, 0.f, dtype, stream);
+}
+
+// h, n_real: a slot whose id is n_real or more adds its weight times the token's own input h.
+SIA_EXPORT int sia_moe_down_ex(const void* act, const void* w2, const int* ids, const float* weights, const void* shared,
+                               const void* shared_gate, int shared_gate_stride, void* out, int n_tokens, int width,
+                               int ff, int top, const void* h, int n_real, int dtype, hipStream_t stream) {
+    if (n_tokens <= 0) return 0;
+    if (width <= 0 || ff <= 0 || top <= 0 || (shared_gate && !shared) || n_real <= 0 || (n_real != 0x7fffffff && !h))
+        return SIA_BAD_ARGUMENT;
+    const int per_block = MOE_WAVES * MOE_PER_WAVE;
+    dim3 grid(n_tokens, (width + per_block - 1) / per_block), block(MOE_WAVES * SIA_WAVE);
+    if (grid.y > 65535) return SIA_BAD_ARGUMENT;
+    const bool vec = ff % 8 == 0;
+    if (dtype == SIA_F32)
+        hipLaunchKernelGGL(moe_down_kernel<float>, grid, block, 0, stream, (const float*)act, (const float*)w2, ids,
+                           weights, (const float*)shared, (const float*)shared_gate, shared_gate_stride, (float*)out,
+                           width, ff, top, vec, (const float*)h, n_real);
+    else if (dtype == SIA_BF16)
+        hipLaunchKernelGGL(moe_down_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)act, (const bf16_t*)w2, ids,
+                           weights, (const bf16_t*)shared, (const bf16_t*)shared_gate, shared_gate_stride, (bf16_t*)out,
+                           width, ff, top, vec, (const bf16_t*)h, n_real);
     else
         return SIA_BAD_ARGUMENT;
     return SIA_LAUNCH_CHECK();
@@ -221,23 +291,8 @@ SIA_EXPORT int sia_moe_gate_up(const void* h, const void* w1, const int* ids, vo
 SIA_EXPORT int sia_moe_down(const void* act, const void* w2, const int* ids, const float* weights, const void* shared,
                             const void* shared_gate, int shared_gate_stride, void* out, int n_tokens, int width, int ff,
                             int top, int dtype, hipStream_t stream) {
-    if (n_tokens <= 0) return 0;
-    if (width <= 0 || ff <= 0 || top <= 0 || (shared_gate && !shared)) return SIA_BAD_ARGUMENT;
-    const int per_block = MOE_WAVES * MOE_PER_WAVE;
-    dim3 grid(n_tokens, (width + per_block - 1) / per_block), block(MOE_WAVES * SIA_WAVE);
-    if (grid.y > 65535) return SIA_BAD_ARGUMENT;
-    const bool vec = ff % 8 == 0;
-    if (dtype == SIA_F32)
-        hipLaunchKernelGGL(moe_down_kernel<float>, grid, block, 0, stream, (const float*)act, (const float*)w2, ids,
-                           weights, (const float*)shared, (const float*)shared_gate, shared_gate_stride, (float*)out,
-                           width, ff, top, vec);
-    else if (dtype == SIA_BF16)
-        hipLaunchKernelGGL(moe_down_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)act, (const bf16_t*)w2, ids,
-                           weights, (const bf16_t*)shared, (const bf16_t*)shared_gate, shared_gate_stride, (bf16_t*)out,
-                           width, ff, top, vec);
-    else
-        return SIA_BAD_ARGUMENT;
-    return SIA_LAUNCH_CHECK();
+    return sia_moe_down_ex(act, w2, ids, weights, shared, shared_gate, shared_gate_stride, out, n_tokens, width, ff, top,
+                           nullptr, 0x7fffffff, dtype, stream);
 }
 
 // ---------------------------------------------------------------------------------------------------------------
@@ -270,8 +325,10 @@ __global__ __launch_bounds__(1024) void moe_sort_kernel(const int* __restrict__ 
     for (int e = threadIdx.x; e < n_experts; e += blockDim.x) count_s[e] = 0;
     for (int i = threadIdx.x; i < max_tiles * MOE_TILE; i += blockDim.x) place_slot[i] = -1;
     __syncthreads();
-    auto expert_of = [&](int s) { return min(max(ids[s], 0), n_experts - 1); };
-    for (int s = threadIdx.x; s < n_slots; s += blockDim.x) atomicAdd(&count_s[expert_of(s)], 1);
+    // a slot whose id lies beyond the experts (an expert without tensors) gets no place: the combine kernel serves it
+    auto expert_of = [&](int s) { return max(ids[s], 0); };
+    for (int s = threadIdx.x; s < n_slots; s += blockDim.x)
+        if (expert_of(s) < n_experts) atomicAdd(&count_s[expert_of(s)], 1);
     __syncthreads();
     if (threadIdx.x == 0) {
         int tile = 0;
@@ -287,7 +344,7 @@ __global__ __launch_bounds__(1024) void moe_sort_kernel(const int* __restrict__ 
     __syncthreads();
     for (int s = threadIdx.x; s < n_slots; s += blockDim.x) {
         const int e = expert_of(s);
-        place_slot[first_s[e] + atomicAdd(&count_s[e], 1)] = s;
+        if (e < n_experts) place_slot[first_s[e] + atomicAdd(&count_s[e], 1)] = s;
     }
 }
 
@@ -299,7 +356,7 @@ __global__ __launch_bounds__(256) void moe_tile_kernel(const bf16_t* __restrict_
                                                        const bf16_t* __restrict__ w, const int* __restrict__ place_slot,
                                                        const int* __restrict__ tile_expert,
                                                        const int* __restrict__ n_tiles, bf16_t* __restrict__ out,
-                                                       int K, int n_out) {
+                                                       int K, int n_out, int glu, float limit) {
     const int tile = blockIdx.x;
     if (tile >= *n_tiles) return;
     const int wave = threadIdx.x / SIA_WAVE, lane = threadIdx.x % SIA_WAVE, r = lane & 15, g = lane >> 4;
@@ -359,7 +416,7 @@ __global__ __launch_bounds__(256) void moe_tile_kernel(const bf16_t* __restrict_
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 float y = acc[nb][mb][0][i];
-                if (GATED) y = y / (1.f + expf(-y)) * acc[nb][mb][1][i];
+                if (GATED) y = gated_activation(y, acc[nb][mb][1][i], glu, limit);
                 v[i] = float_to_bf16(y);
             }
             bf16_t* dst = out + row * n_out + c;
@@ -378,14 +435,19 @@ __global__ __launch_bounds__(256) void moe_tile_kernel(const bf16_t* __restrict_
 __global__ __launch_bounds__(256) void moe_combine_kernel(const bf16_t* __restrict__ y, const float* __restrict__ weights,
                                                           const bf16_t* __restrict__ shared,
                                                           const bf16_t* __restrict__ shared_gate, int shared_gate_stride,
-                                                          bf16_t* __restrict__ out, int width, int top) {
+                                                          bf16_t* __restrict__ out, int width, int top,
+                                                          const int* __restrict__ ids, const bf16_t* __restrict__ h,
+                                                          int n_real) {
     const int n = blockIdx.x;
     float scale = 1.f;
     if (shared && shared_gate) scale = 1.f / (1.f + expf(-bf16_to_float(shared_gate[(size_t)n * shared_gate_stride])));
     for (int c = threadIdx.x; c < width; c += blockDim.x) {
         float acc = 0.f;
-        for (int k = 0; k < top; ++k)
-            acc += weights[(size_t)n * top + k] * bf16_to_float(y[((size_t)n * top + k) * width + c]);
+        for (int k = 0; k < top; ++k) {
+            const size_t slot = (size_t)n * top + k;
+            // an expert without tensors returns the token's input; its row of y was never written
+            acc += weights[slot] * bf16_to_float(ids[slot] >= n_real ? h[(size_t)n * width + c] : y[slot * width + c]);
+        }
         if (shared) acc += scale * bf16_to_float(shared[(size_t)n * width + c]);
         out[(size_t)n * width + c] = float_to_bf16(acc);
     }
@@ -401,13 +463,14 @@ SIA_EXPORT long long sia_moe_tiled_workspace(int n_tokens, int top, int n_expert
 }
 
 // act [slots, ff] and y [slots, width] are the caller's scratch (bfloat16).
-SIA_EXPORT int sia_moe_tiled(const void* h, const void* w1, const void* w2, const int* ids, const float* weights,
-                             const void* shared, const void* shared_gate, int shared_gate_stride, void* act, void* y,
-                             void* out, int* workspace, int n_tokens, int width, int ff, int top, int n_experts,
-                             hipStream_t stream) {
+// glu, limit: the experts' gated activation; ids of n_experts and more name experts without tensors.
+SIA_EXPORT int sia_moe_tiled_ex(const void* h, const void* w1, const void* w2, const int* ids, const float* weights,
+                                const void* shared, const void* shared_gate, int shared_gate_stride, void* act, void* y,
+                                void* out, int* workspace, int n_tokens, int width, int ff, int top, int n_experts,
+                                int glu, float limit, hipStream_t stream) {
     if (n_tokens <= 0) return 0;
     if (sia_moe_tiled_workspace(n_tokens, top, n_experts, width, ff) == 0 || n_experts > MOE_MAX_EXPERTS ||
-        (shared_gate && !shared))
+        (shared_gate && !shared) || (glu != SIA_GLU_SILU && glu != SIA_GLU_CLAMPED))
         return SIA_BAD_ARGUMENT;
     const int slots = n_tokens * top;
     const int max_tiles = (slots + MOE_TILE - 1) / MOE_TILE + n_experts;
@@ -417,10 +480,21 @@ SIA_EXPORT int sia_moe_tiled(const void* h, const void* w1, const void* w2, cons
     hipLaunchKernelGGL(moe_sort_kernel, dim3(1), dim3(1024), 0, stream, ids, slots, n_experts, place_slot, tile_expert,
                        n_tiles, max_tiles);
     hipLaunchKernelGGL(moe_tile_kernel<true>, dim3(max_tiles, (ff + 127) / 128), dim3(256), 0, stream,
-                       (const bf16_t*)h, top, (const bf16_t*)w1, place_slot, tile_expert, n_tiles, (bf16_t*)act, width, ff);
+                       (const bf16_t*)h, top, (const bf16_t*)w1, place_slot, tile_expert, n_tiles, (bf16_t*)act, width, ff,
+                       glu, limit);
     hipLaunchKernelGGL(moe_tile_kernel<false>, dim3(max_tiles, (width + 127) / 128), dim3(256), 0, stream,
-                       (const bf16_t*)act, 1, (const bf16_t*)w2, place_slot, tile_expert, n_tiles, (bf16_t*)y, ff, width);
+                       (const bf16_t*)act, 1, (const bf16_t*)w2, place_slot, tile_expert, n_tiles, (bf16_t*)y, ff, width,
+                       SIA_GLU_SILU, 0.f);
     hipLaunchKernelGGL(moe_combine_kernel, dim3(n_tokens), dim3(256), 0, stream, (const bf16_t*)y, weights,
-                       (const bf16_t*)shared, (const bf16_t*)shared_gate, shared_gate_stride, (bf16_t*)out, width, top);
+                       (const bf16_t*)shared, (const bf16_t*)shared_gate, shared_gate_stride, (bf16_t*)out, width, top,
+                       ids, (const bf16_t*)h, n_experts);
     return SIA_LAUNCH_CHECK();
+}
+
+SIA_EXPORT int sia_moe_tiled(const void* h, const void* w1, const void* w2, const int* ids, const float* weights,
+                             const void* shared, const void* shared_gate, int shared_gate_stride, void* act, void* y,
+                             void* out, int* workspace, int n_tokens, int width, int ff, int top, int n_experts,
+                             hipStream_t stream) {
+    return sia_moe_tiled_ex(h, w1, w2, ids, weights, shared, shared_gate, shared_gate_stride, act, y, out, workspace,
+                            n_tokens, width, ff, top, n_experts, SIA_GLU_SILU, 0.f, stream);
 }

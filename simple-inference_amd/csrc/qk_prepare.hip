@@ -93,7 +93,7 @@ __global__ __launch_bounds__(QKP_WAVES* SIA_WAVE) void qk_prepare_kernel(
     const int* __restrict__ block_table, int table_width, T* __restrict__ k_pages, T* __restrict__ v_pages,
     int n_tokens, int n_heads, int n_kv, int head_dim, int value_dim, int rotary_dim, int page_size, int v_group,
     int k_row, int v_rows, T* q_out, int q_row_stride, int q_head_stride, float temp_coef,
-    int temp_every) {   // q_out may be qkv
+    int temp_every, int values_are_keys) {   // q_out may be qkv
     const int n = blockIdx.x, wave = threadIdx.x / SIA_WAVE, lane = threadIdx.x % SIA_WAVE;
     const int pos = positions[n];
     const int half = rotary_dim / 2;
@@ -102,7 +102,8 @@ __global__ __launch_bounds__(QKP_WAVES* SIA_WAVE) void qk_prepare_kernel(
         page = block_table[(size_t)seq_of_token[n] * table_width + pos / page_size];
         off = pos % page_size;
     }
-    const int k_first = n_heads * head_dim, v_first = k_first + n_kv * head_dim;
+    // values that are the keys as projected: the value rows are read from the k columns, and the row has no v columns
+    const int k_first = n_heads * head_dim, v_first = values_are_keys ? k_first : k_first + n_kv * head_dim;
     const int qk_groups = (n_heads + n_kv + QKP_WAVES - 1) / QKP_WAVES;
     if ((int)blockIdx.y >= qk_groups) {  // the token's values
         if (page >= 0)
@@ -177,12 +178,13 @@ __global__ __launch_bounds__(QKP_WAVES* SIA_WAVE) void qk_prepare_vec_kernel(
     const int* __restrict__ block_table, int table_width, T* __restrict__ k_pages, T* __restrict__ v_pages,
     int n_tokens, int n_heads, int n_kv, int head_dim, int value_dim, int rotary_dim, int page_size, int v_group,
     int k_row, int v_rows, T* q_out, int q_row_stride, int q_head_stride, float temp_coef,
-    int temp_every) {   // q_out may be qkv
+    int temp_every, int values_are_keys) {   // q_out may be qkv
     const int n = blockIdx.x, wave = threadIdx.x / SIA_WAVE, lane = threadIdx.x % SIA_WAVE;
     const int pos = positions[n];
     const int half = rotary_dim / 2;
     const int group = head_dim / 8, heads_a_wave = SIA_WAVE / group;   // lanes of a head; a power of two up to 32
-    const int k_first = n_heads * head_dim, v_first = k_first + n_kv * head_dim;
+    // values that are the keys as projected: the value rows are read from the k columns, and the row has no v columns
+    const int k_first = n_heads * head_dim, v_first = values_are_keys ? k_first : k_first + n_kv * head_dim;
     const int qk_groups = (n_heads + n_kv + QKP_WAVES * heads_a_wave - 1) / (QKP_WAVES * heads_a_wave);
     if ((int)blockIdx.y >= qk_groups) {  // the token's values
         const int page = block_table[(size_t)seq_of_token[n] * table_width + pos / page_size];
@@ -255,19 +257,23 @@ __global__ __launch_bounds__(QKP_WAVES* SIA_WAVE) void qk_prepare_vec_kernel(
 
 SIA_EXPORT int sia_qk_prepare_max_head_dim() { return QKP_MAX_HEAD_DIM; }
 
-SIA_EXPORT int sia_qk_prepare(void* qkv, int row_stride, const float* bias, const float* q_gain, const float* k_gain,
-                              float eps, const float* cos_table, const float* sin_table, const int* positions,
-                              const int* seq_of_token, const int* block_table, int table_width, void* k_pages,
-                              void* v_pages, int n_tokens, int n_heads, int n_kv, int head_dim, int value_dim,
-                              int rotary_dim, int page_size, int k_row, int v_rows, void* q_out, int q_row_stride,
-                              int q_head_stride, float temp_coef, int temp_every, int dtype, hipStream_t stream) {
+// values_are_keys: the row is [q heads | k heads] and a position's value rows are its k heads as projected (with
+// their bias, before norm and rotation); value_dim is then head_dim.
+SIA_EXPORT int sia_qk_prepare_ex(void* qkv, int row_stride, const float* bias, const float* q_gain, const float* k_gain,
+                                 float eps, const float* cos_table, const float* sin_table, const int* positions,
+                                 const int* seq_of_token, const int* block_table, int table_width, void* k_pages,
+                                 void* v_pages, int n_tokens, int n_heads, int n_kv, int head_dim, int value_dim,
+                                 int rotary_dim, int page_size, int k_row, int v_rows, void* q_out, int q_row_stride,
+                                 int q_head_stride, float temp_coef, int temp_every, int values_are_keys, int dtype,
+                                 hipStream_t stream) {
     if (n_tokens <= 0) return 0;
+    if (values_are_keys && value_dim != head_dim) return SIA_BAD_ARGUMENT;
     if (head_dim <= 0 || head_dim > QKP_MAX_HEAD_DIM || value_dim <= 0 || n_heads < 0 || n_kv < 0) return SIA_BAD_ARGUMENT;
     if (rotary_dim < 0 || rotary_dim > head_dim || (rotary_dim & 1)) return SIA_BAD_ARGUMENT;
     if (rotary_dim > 0 && (!cos_table || !sin_table)) return SIA_BAD_ARGUMENT;
     if ((q_gain == nullptr) != (k_gain == nullptr)) return SIA_BAD_ARGUMENT;
     if (n_kv > 0 && (!k_pages || !v_pages || !block_table || page_size <= 0)) return SIA_BAD_ARGUMENT;
-    if (row_stride < n_heads * head_dim + n_kv * (head_dim + value_dim)) return SIA_BAD_ARGUMENT;
+    if (row_stride < n_heads * head_dim + n_kv * (head_dim + (values_are_keys ? 0 : value_dim))) return SIA_BAD_ARGUMENT;
     if (n_kv > 0 && (k_row < head_dim || v_rows < value_dim)) return SIA_BAD_ARGUMENT;
     if (!q_out) {  // q goes back where it came from
         q_out = qkv;
@@ -290,17 +296,29 @@ SIA_EXPORT int sia_qk_prepare(void* qkv, int row_stride, const float* bias, cons
                                k_gain, eps, cos_table, sin_table, positions, seq_of_token, block_table, table_width, \
                                (T*)k_pages, (T*)v_pages, n_tokens, n_heads, n_kv, head_dim, value_dim, rotary_dim,   \
                                page_size, v_group, k_row, v_rows, (T*)q_out, q_row_stride, q_head_stride, temp_coef,  \
-                               temp_every);                                                                          \
+                               temp_every, values_are_keys);                                                                       \
         else                                                                                                         \
             hipLaunchKernelGGL(qk_prepare_kernel<T>, grid, block, 0, stream, (T*)qkv, row_stride, bias, q_gain,      \
                                k_gain, eps, cos_table, sin_table, positions, seq_of_token, block_table, table_width, \
                                (T*)k_pages, (T*)v_pages, n_tokens, n_heads, n_kv, head_dim, value_dim, rotary_dim,   \
                                page_size, v_group, k_row, v_rows, (T*)q_out, q_row_stride, q_head_stride, temp_coef,  \
-                               temp_every);                                                                          \
+                               temp_every, values_are_keys);                                                                       \
     } while (0)
     if (dtype == SIA_F32) LAUNCH(float);
     else if (dtype == SIA_BF16) LAUNCH(bf16_t);
     else return SIA_BAD_ARGUMENT;
 #undef LAUNCH
     return SIA_LAUNCH_CHECK();
+}
+
+SIA_EXPORT int sia_qk_prepare(void* qkv, int row_stride, const float* bias, const float* q_gain, const float* k_gain,
+                              float eps, const float* cos_table, const float* sin_table, const int* positions,
+                              const int* seq_of_token, const int* block_table, int table_width, void* k_pages,
+                              void* v_pages, int n_tokens, int n_heads, int n_kv, int head_dim, int value_dim,
+                              int rotary_dim, int page_size, int k_row, int v_rows, void* q_out, int q_row_stride,
+                              int q_head_stride, float temp_coef, int temp_every, int dtype, hipStream_t stream) {
+    return sia_qk_prepare_ex(qkv, row_stride, bias, q_gain, k_gain, eps, cos_table, sin_table, positions, seq_of_token,
+                             block_table, table_width, k_pages, v_pages, n_tokens, n_heads, n_kv, head_dim, value_dim,
+                             rotary_dim, page_size, k_row, v_rows, q_out, q_row_stride, q_head_stride, temp_coef,
+                             temp_every, 0, dtype, stream);
 }

@@ -674,3 +674,243 @@ SIA_EXPORT int sia_ssd_scan(const void* proj, int row_stride, const void* xbc, i
 #undef RUN
     return SIA_LAUNCH_CHECK();
 }
+
+// ---------------------------------------------------------------------------------------------------------------
+// Linear attention with a constant decay per head, behind activations:
+//   q, k, v = silu(z_q), silu(z_k), silu(z_v);  S <- decay_h S + k v^T;  o = S^T q                  S [D, Dv] per head
+//   out = o / sqrt(mean over the whole row of o^2 + eps) * w * sigmoid(z_g)                          w [H * Dv]
+// Rows are [z_q (H * D) | z_k (H * D) | z_v (H * Dv) | z_g (H * Dv)].  A first kernel leaves the activations in the
+// rows' own columns and the decays, one per head, in the float workspace as the recurrence reads them; then the
+// recurrence above with raw outputs, and a kernel that norms a row over all its heads and gates it.
+template <typename T>
+__global__ __launch_bounds__(256) void decay_prepare_kernel(T* __restrict__ proj, int row_stride,
+                                                            const float* __restrict__ decays,
+                                                            float* __restrict__ alpha, int n_heads, int D, int active) {
+    const int n = blockIdx.x, c = blockIdx.y * blockDim.x + threadIdx.x;
+    if (c < active) {
+        T* row = proj + (size_t)n * row_stride;
+        const float z = to_float(row[c]);
+        row[c] = from_float<T>(z / (1.f + expf(-z)));
+    }
+    if (c < n_heads * D) alpha[(size_t)n * n_heads * D + c] = decays[c / D];
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void decay_finish_kernel(const float* __restrict__ raw, const T* __restrict__ proj,
+                                                           int row_stride, int g_col,
+                                                           const float* __restrict__ norm_w, T* __restrict__ out,
+                                                           int inner, float eps) {
+    __shared__ float scratch[16];
+    const int n = blockIdx.x;
+    const float* o = raw + (size_t)n * inner;
+    const T* g = proj + (size_t)n * row_stride + g_col;
+    float ss = 0.f;
+    for (int c = threadIdx.x; c < inner; c += blockDim.x) ss += o[c] * o[c];
+    const float inv = rsqrtf(block_sum(ss, scratch) / (float)inner + eps);
+    for (int c = threadIdx.x; c < inner; c += blockDim.x) {
+        const float z = to_float(g[c]);
+        out[(size_t)n * inner + c] = from_float<T>(o[c] * inv * norm_w[c] * (1.f / (1.f + expf(-z))));
+    }
+}
+
+SIA_EXPORT int sia_decay_attention(void* proj, int row_stride, const float* decays, const float* norm_w, float* state,
+                                   const int* cu_q, const int* slots, void* out, int n_tokens, int n_seqs,
+                                   int max_q_len, int n_heads, int D, int Dv, float eps, int dtype, float* workspace,
+                                   hipStream_t stream) {
+    if (n_seqs <= 0 || n_tokens <= 0) return 0;
+    if (D <= 0 || Dv <= 0 || D > 512 || Dv > 512 || n_heads <= 0 || n_heads > 65535 || !state || !norm_w || !decays ||
+        !workspace || row_stride < n_heads * (2 * D + 2 * Dv))
+        return SIA_BAD_ARGUMENT;
+    const int qk = n_heads * D, inner = n_heads * Dv, active = 2 * qk + inner;
+    float* alpha = workspace;
+    float* raw_space = alpha + (size_t)n_tokens * qk;
+    dim3 pgrid(n_tokens, (active + 255) / 256), pblock(256), fgrid(n_tokens), fblock(256);
+    bool raw = false;
+#define RUN(T)                                                                                                          \
+    do {                                                                                                                \
+        hipLaunchKernelGGL(decay_prepare_kernel<T>, pgrid, pblock, 0, stream, (T*)proj, row_stride, decays, alpha,      \
+                           n_heads, D, active);                                                                         \
+        const int code = launch_recurrence(proj, row_stride, 0, qk, 2 * qk, -1, nullptr, 1, alpha, norm_w, state,       \
+                                           (long long)n_heads * D * Dv, cu_q, slots, nullptr, n_seqs, max_q_len,        \
+                                           n_heads, D, Dv, 1.f, eps, dtype, raw_space, true, &raw, stream);             \
+        if (code) return code;                                                                                          \
+        hipLaunchKernelGGL(decay_finish_kernel<T>, fgrid, fblock, 0, stream, raw_space, (const T*)proj, row_stride,     \
+                           active, norm_w, (T*)out, inner, eps);                                                        \
+    } while (0)
+    if (dtype == SIA_F32) RUN(float);
+    else if (dtype == SIA_BF16) RUN(bf16_t);
+    else return SIA_BAD_ARGUMENT;
+#undef RUN
+    return SIA_LAUNCH_CHECK();
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// The gated delta rule, token by token:
+//   q <- q / sqrt(sum(q^2) + 1e-6) * D^(-1/2),  k <- k / sqrt(sum(k^2) + 1e-6)            per query/key head
+//   beta = sigmoid(z_b),  g = exp(-exp(A_log_h) * softplus(z_a + dt_bias_h))              per value head
+//   S <- g S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q                          S [D, Dv] per value head
+//   out = o * rsqrt(mean(o^2) + eps) * w * silu(z_g)                                      per head, w [Dv]
+// q, k [G * D] and v [H * Dv] are columns of the convolved rows (value head h reads query/key head h / (H / G)); z_g
+// [H * Dv], z_b and z_a [H] are columns of the projected rows.  A workgroup owns a (sequence, value head) or, in a
+// step of few such pairs and many tokens, a slice of the head's columns (a column of S is corrected and read alone:
+// S^T k and S^T q are sums down a column).  Thread (j, r) keeps rows r, r + R, ... of column j in registers; a token
+// costs two sums over the R lanes of a column, one before the write and one after.  Blocks of tokens are staged
+// through LDS as floats, where the unit norms, the write strengths and the decays of the block are taken, by every
+// workgroup for itself.  The raw outputs go to the float workspace; the head's norm and gate are a second kernel.
+template <typename T, int ROWS>
+__global__ __launch_bounds__(512) void delta_rule_kernel(
+    const T* __restrict__ qkv, int qkv_stride, const T* __restrict__ proj, int proj_stride, int b_col, int a_col,
+    const float* __restrict__ a_log, const float* __restrict__ dt_bias, float* __restrict__ state,
+    long long state_stride, const int* __restrict__ cu_q, const int* __restrict__ slots, float* __restrict__ raw_out,
+    int n_heads, int n_kv, int D, int Dv, int R, int block_tokens, int slice) {
+    extern __shared__ float lds[];
+    const int seq = blockIdx.x, head = blockIdx.y, tid = threadIdx.x;
+    const int j0 = blockIdx.z * slice;
+    const int first = cu_q[seq], last = cu_q[seq + 1];
+    if (first >= last) return;
+    const int TB = block_tokens;
+    float* q_s = lds;                  // [TB][D]
+    float* k_s = q_s + TB * D;         // [TB][D]
+    float* v_s = k_s + TB * D;         // [TB][slice]
+    float* be_s = v_s + TB * slice;    // [TB]
+    float* de_s = be_s + TB;           // [TB]
+    const int j = j0 + tid / R, r = tid % R;
+    const bool owns = tid / R < slice && j < Dv;
+    float* S_mem = state + (size_t)slots[seq] * state_stride + (size_t)head * D * Dv;
+    float S[ROWS];
+#pragma unroll
+    for (int i = 0; i < ROWS; ++i) {
+        const int d = i * R + r;
+        S[i] = (owns && d < D) ? S_mem[(size_t)d * Dv + j] : 0.f;
+    }
+    const int wave = tid / SIA_WAVE, lane = tid % SIA_WAVE, n_waves = blockDim.x / SIA_WAVE;
+    const int kv_head = head / (n_heads / n_kv);
+    const int q_col = kv_head * D, k_col = n_kv * D + kv_head * D, v_col = 2 * n_kv * D + head * Dv;
+    const float rate = expf(a_log[head]), bias = dt_bias ? dt_bias[head] : 0.f;
+    const float q_scale = rsqrtf((float)D);
+
+    for (int t0 = first; t0 < last; t0 += TB) {
+        const int nt = min(TB, last - t0);
+        for (int idx = tid; idx < nt * slice; idx += blockDim.x) {
+            const int t = idx / slice, c = idx % slice;
+            v_s[idx] = j0 + c < Dv ? to_float(qkv[(size_t)(t0 + t) * qkv_stride + v_col + j0 + c]) : 0.f;
+        }
+        for (int idx = tid; idx < nt * D; idx += blockDim.x) {
+            const int t = idx / D, c = idx % D;
+            const T* row = qkv + (size_t)(t0 + t) * qkv_stride;
+            q_s[idx] = to_float(row[q_col + c]);
+            k_s[idx] = to_float(row[k_col + c]);
+        }
+        if (tid < nt) {
+            const T* row = proj + (size_t)(t0 + tid) * proj_stride;
+            const float zb = to_float(row[b_col + head]), za = to_float(row[a_col + head]) + bias;
+            be_s[tid] = 1.f / (1.f + expf(-zb));
+            de_s[tid] = expf(-rate * (fmaxf(za, 0.f) + log1pf(expf(-fabsf(za)))));
+        }
+        __syncthreads();
+        for (int t = wave; t < nt; t += n_waves) {      // unit vectors, a wave a token
+            float sq = 0.f, sk = 0.f;
+            for (int c = lane; c < D; c += SIA_WAVE) {
+                sq += q_s[t * D + c] * q_s[t * D + c];
+                sk += k_s[t * D + c] * k_s[t * D + c];
+            }
+            const float iq = rsqrtf(wave_sum(sq) + 1e-6f) * q_scale, ik = rsqrtf(wave_sum(sk) + 1e-6f);
+            for (int c = lane; c < D; c += SIA_WAVE) {
+                q_s[t * D + c] *= iq;
+                k_s[t * D + c] *= ik;
+            }
+        }
+        __syncthreads();
+        for (int t = 0; t < nt; ++t) {
+            const float g = de_s[t], b = be_s[t];
+            const float v = owns ? v_s[t * slice + (j - j0)] : 0.f;
+            float kept = 0.f;
+#pragma unroll
+            for (int i = 0; i < ROWS; ++i) {
+                const int d = i * R + r;
+                if (d < D) {
+                    S[i] *= g;
+                    kept += k_s[t * D + d] * S[i];
+                }
+            }
+            for (int o = R / 2; o > 0; o >>= 1) kept += __shfl_xor(kept, o, SIA_WAVE);
+            const float u = b * (v - kept);
+            float acc = 0.f;
+#pragma unroll
+            for (int i = 0; i < ROWS; ++i) {
+                const int d = i * R + r;
+                if (d < D) {
+                    S[i] += k_s[t * D + d] * u;
+                    acc += q_s[t * D + d] * S[i];
+                }
+            }
+            for (int o = R / 2; o > 0; o >>= 1) acc += __shfl_xor(acc, o, SIA_WAVE);
+            if (owns && r == 0) raw_out[((size_t)(t0 + t) * n_heads + head) * Dv + j] = acc;
+        }
+        __syncthreads();
+    }
+#pragma unroll
+    for (int i = 0; i < ROWS; ++i) {
+        const int d = i * R + r;
+        if (owns && d < D) S_mem[(size_t)d * Dv + j] = S[i];
+    }
+}
+
+// floats of workspace: the raw outputs [tokens, heads, Dv]
+SIA_EXPORT long long sia_delta_rule_workspace(int n_tokens, int n_heads, int Dv) {
+    return (long long)n_tokens * n_heads * Dv;
+}
+
+SIA_EXPORT int sia_delta_rule(const void* qkv, int qkv_stride, const void* proj, int proj_stride, int g_col, int b_col,
+                              int a_col, const float* a_log, const float* dt_bias, const float* norm_w, float* state,
+                              long long state_stride, const int* cu_q, const int* slots, void* out, int n_tokens,
+                              int n_seqs, int max_q_len, int n_heads, int n_kv, int D, int Dv, float eps, int dtype,
+                              float* workspace, hipStream_t stream) {
+    if (n_seqs <= 0 || n_tokens <= 0) return 0;
+    if (D <= 0 || Dv <= 0 || D > 512 || Dv > 512 || n_heads <= 0 || n_heads > 65535 || n_kv <= 0 || n_heads % n_kv ||
+        !state || !norm_w || !a_log || !workspace || qkv_stride < 2 * n_kv * D + n_heads * Dv || g_col < 0 ||
+        b_col < 0 || a_col < 0 || g_col + n_heads * Dv > proj_stride || b_col + n_heads > proj_stride ||
+        a_col + n_heads > proj_stride || state_stride < (long long)n_heads * D * Dv)
+        return SIA_BAD_ARGUMENT;
+    // columns a workgroup: all of a head's, or in a step of runs of tokens a slice of them, as narrow as it takes to
+    // fill the chip; lanes a column: the largest power of two that keeps the workgroup within 512 threads
+    int slice = Dv;
+    if (max_q_len > 1)
+        while (slice > 8 && (long long)n_seqs * n_heads * ((Dv + slice - 1) / slice) < 256) slice = (slice + 1) / 2;
+    int R = 1, rows = D;
+    for (;;) {
+        R = 1;
+        while (R * 2 <= SIA_WAVE && slice * R * 2 <= 512 && R * 2 <= D) R *= 2;
+        rows = (D + R - 1) / R;
+        if (rows <= 128 || slice <= 1) break;
+        slice = (slice + 1) / 2;
+    }
+    if (rows > 128) return SIA_BAD_ARGUMENT;
+    const int threads = ((slice * R + SIA_WAVE - 1) / SIA_WAVE) * SIA_WAVE;
+    int TB = max_q_len >= 16 ? 16 : (max_q_len >= 4 ? 4 : 1);
+    auto bytes = [&](int tb) { return (size_t)tb * (2 * D + slice + 2) * sizeof(float); };
+    while (TB > 1 && bytes(TB) > 60 * 1024) TB /= 2;
+    if (bytes(TB) > 60 * 1024) return SIA_BAD_ARGUMENT;
+    dim3 grid(n_seqs, n_heads, (Dv + slice - 1) / slice), block(threads), fgrid(n_tokens, n_heads), fblock(SIA_WAVE);
+#define LAUNCH(T, ROWS)                                                                                              \
+    hipLaunchKernelGGL((delta_rule_kernel<T, ROWS>), grid, block, bytes(TB), stream, (const T*)qkv, qkv_stride,      \
+                       (const T*)proj, proj_stride, b_col, a_col, a_log, dt_bias, state, state_stride, cu_q, slots,   \
+                       workspace, n_heads, n_kv, D, Dv, R, TB, slice)
+#define RUN(T)                                                                                                       \
+    do {                                                                                                             \
+        if (rows <= 4) LAUNCH(T, 4);                                                                                 \
+        else if (rows <= 8) LAUNCH(T, 8);                                                                            \
+        else if (rows <= 16) LAUNCH(T, 16);                                                                          \
+        else if (rows <= 32) LAUNCH(T, 32);                                                                          \
+        else if (rows <= 64) LAUNCH(T, 64);                                                                          \
+        else LAUNCH(T, 128);                                                                                         \
+        hipLaunchKernelGGL(gla_finish_kernel<T>, fgrid, fblock, 0, stream, workspace, (const T*)proj, proj_stride,   \
+                           g_col, norm_w, (T*)out, n_heads, Dv, eps);                                                \
+    } while (0)
+    if (dtype == SIA_F32) RUN(float);
+    else if (dtype == SIA_BF16) RUN(bf16_t);
+    else return SIA_BAD_ARGUMENT;
+#undef RUN
+#undef LAUNCH
+    return SIA_LAUNCH_CHECK();
+}

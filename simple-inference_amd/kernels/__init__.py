@@ -22,7 +22,8 @@ import torch
 from . import build
 
 _DT = {torch.float32: 0, torch.bfloat16: 1}
-_ACTIVATIONS = {"relu2": 0, "gelu_tanh": 1}   # ``SiaActivation`` of csrc/common.h
+_ACTIVATIONS = {"relu2": 0, "gelu_tanh": 1, "gelu": 2}   # ``SiaActivation`` of csrc/common.h
+_GLUS = {"silu": 0, "clamped": 1}                        # ``SiaGlu`` of csrc/common.h
 
 _c_int, _c_float, _c_ptr, _c_ll = ctypes.c_int, ctypes.c_float, ctypes.c_void_p, ctypes.c_longlong
 
@@ -101,6 +102,26 @@ _SIGNATURES = {
     "sia_place_tokens": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr],
     "sia_scale_rows": [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_float, _c_ptr],
     "sia_stream_read": [_c_ptr, _c_ll, _c_ptr, _c_ptr],
+    "sia_add_rmsnorm_scaled": [_c_ptr, _c_ptr, _c_float, _c_ptr, _c_float, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_float,
+                               _c_int, _c_ptr],
+    "sia_scaled_sum": [_c_ptr, _c_float, _c_ptr, _c_float, _c_ptr, _c_ll, _c_int, _c_ptr],
+    "sia_glu": [_c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_float, _c_int, _c_ptr],
+    "sia_qk_prepare_ex": [_c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_float, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int,
+                          _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr,
+                          _c_int, _c_int, _c_float, _c_int, _c_int, _c_int, _c_ptr],
+    "sia_decay_attention": [_c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int,
+                            _c_int, _c_int, _c_float, _c_int, _c_ptr, _c_ptr],
+    "sia_delta_rule_workspace": [_c_int, _c_int, _c_int],
+    "sia_delta_rule": [_c_ptr, _c_int, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ll, _c_ptr,
+                       _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_ptr,
+                       _c_ptr],
+    "sia_moe_route_corrected": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr],
+    "sia_moe_gate_up_ex": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int,
+                           _c_ptr],
+    "sia_moe_down_ex": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_int, _c_int, _c_int, _c_int,
+                        _c_ptr, _c_int, _c_int, _c_ptr],
+    "sia_moe_tiled_ex": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
+                         _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_ptr],
 }
 
 
@@ -208,6 +229,7 @@ class HipKernels:
         self.core.sia_moe_tiled_workspace.restype = ctypes.c_longlong
         self.core.sia_hgrn2_workspace.restype = ctypes.c_longlong
         self.core.sia_ssd_workspace.restype = ctypes.c_longlong
+        self.core.sia_delta_rule_workspace.restype = ctypes.c_longlong
         self.tiled_experts = True        # many slots in bfloat16: experts' products on the matrix cores, slots sorted by expert
         self._attn_libs = {}
         # the short way to the current stream's handle, where this torch has it (a few microseconds less a launch)
@@ -364,12 +386,16 @@ class HipKernels:
 
     # -- residual add + rms norm ---------------------------------------------
     def add_rmsnorm(self, residual, delta, weight, eps, out_dtype, rows=None, gate=None, gate_bias=None,
-                    delta_bias=None):
+                    delta_bias=None, terms=None):
         """``residual += delta`` and the RMS norm of the sum.  With ``gate`` (the logits of an elementwise gate:
         ``[n, hidden]``, which may be columns of a wider matrix) the sum is
-        ``residual += (delta + delta_bias) * sigmoid(gate + gate_bias)``."""
+        ``residual += (delta + delta_bias) * sigmoid(gate + gate_bias)``.  With ``terms`` (``[(tensor, factor)]``, in
+        place of ``delta``) the sum is ``residual += sum_i factor_i * tensor_i``; without a ``weight`` only that sum is
+        made and nothing returned."""
         n, hidden = residual.shape
         self._want(residual, "residual", torch.float32)
+        if terms is not None:
+            return self._add_terms(residual, terms, weight, eps, out_dtype, rows)
         self._want(weight, "norm weight", torch.float32, (hidden,))
         if out_dtype not in _DT:
             raise KernelError(f"norm output dtype {out_dtype} is not float32 or bfloat16")
@@ -388,6 +414,50 @@ class HipKernels:
                                               n_out, hidden, float(eps), _DT[out_dtype], self._stream()),
                     "add_rmsnorm")
         return out
+
+    def _add_terms(self, residual, terms, weight, eps, out_dtype, rows):
+        n, hidden = residual.shape
+        terms = list(terms)
+        if not terms:
+            raise KernelError("a sum of scaled terms needs at least one (tensor, factor) pair")
+        dtype = terms[0][0].dtype
+        if dtype not in _DT or (weight is not None and out_dtype != dtype):
+            raise KernelError(f"scaled terms are float32 or bfloat16 and of the norm's output type, got {dtype}")
+        for y, _ in terms:
+            self._want(y, "scaled term", dtype, (n, hidden))
+        if len(terms) > 2:      # the kernel takes two: what is beyond is added up beforehand
+            terms = [(self.scaled_sum(terms[:-1]), 1.0), terms[-1]]
+        (d1, f1), (d2, f2) = terms[0], (terms[1] if len(terms) > 1 else (None, 0.0))
+        n_out, out = n, None
+        if rows is not None:
+            self._want(rows, "rows", torch.int32)
+            n_out = rows.numel()
+        if weight is not None:
+            self._want(weight, "norm weight", torch.float32, (hidden,))
+            out = torch.empty((n_out, hidden), dtype=dtype, device=residual.device)
+        elif rows is not None:
+            raise KernelError("a sum alone is made over all rows")
+        self._check(self.core.sia_add_rmsnorm_scaled(_ptr(residual), _ptr(d1), float(f1), _ptr(d2), float(f2), _ptr(weight),
+                                                     _ptr(out), _ptr(rows), n_out, hidden, float(eps), _DT[dtype],
+                                                     self._stream()), "add_rmsnorm_scaled")
+        return out
+
+    def scaled_sum(self, terms):
+        """``sum_i factor_i * tensor_i`` in float, rounded to the tensors' type."""
+        terms = list(terms)
+        first = terms[0][0]
+        if first.dtype not in _DT:
+            raise KernelError(f"scaled terms are float32 or bfloat16, got {first.dtype}")
+        for y, _ in terms:
+            self._want(y, "scaled term", first.dtype, tuple(first.shape))
+        total, factor = first, float(terms[0][1])
+        rest = terms[1:] or [(None, 0.0)]
+        for y, f in rest:
+            out = torch.empty_like(first)
+            self._check(self.core.sia_scaled_sum(_ptr(total), factor, _ptr(y), float(f), _ptr(out), first.numel(),
+                                                 _DT[first.dtype], self._stream()), "scaled_sum")
+            total, factor = out, 1.0
+        return total
 
     def gated_add(self, residual, delta, gate=None, gate_bias=None, delta_bias=None):
         """``residual += (delta + delta_bias) * sigmoid(gate + gate_bias)`` and nothing else (without ``gate`` the
@@ -516,15 +586,17 @@ class HipKernels:
             raise KernelError(f"head sizes {key_dim} x {value_dim} are outside what the recurrent kernel takes (up to {limit})")
 
     # -- mixture of experts ------------------------------------------------------------
-    def moe_route(self, h, router, top, score="softmax", groups=None, scale=1.0):
+    def moe_route(self, h, router, top, score="softmax", groups=None, scale=1.0, correction=None):
         """The ``top`` experts of every row with the largest router logits ``h @ router^T`` (float; ties go to the
         lower index) and the softmax over their logits alone: ``(ids [n, top] int32, weights [n, top] float32)``.
         ``score="sigmoid"``: the scores are the logits' sigmoids; with ``groups = (count, keep)`` only experts of the
         ``keep`` groups (of ``count`` equal groups of neighbours) whose two largest scores sum highest can be chosen;
         the weights are the chosen scores over their sum, times ``scale``."""
-        if score not in ("softmax", "sigmoid"):
-            raise KernelError(f"score must be 'softmax' or 'sigmoid', got {score!r}")
-        if score == "softmax" and (groups is not None or scale != 1.0):
+        if score not in ("softmax", "sigmoid", "softmax_all"):
+            raise KernelError(f"score must be 'softmax', 'sigmoid' or 'softmax_all', got {score!r}")
+        if correction is not None and score != "softmax_all":
+            raise KernelError("a correction of the choice comes with scores over all experts")
+        if score != "sigmoid" and (groups is not None or scale != 1.0):
             raise KernelError("expert groups and a scale on the weights come with sigmoid scores")
         self._want(h, "router input")
         n, width = h.shape
@@ -539,6 +611,14 @@ class HipKernels:
             raise KernelError(f"{experts} experts in {count} groups of which {keep} are kept cannot give {top}")
         if not 0 < top <= experts:
             raise KernelError(f"top {top} is not between 1 and the number of experts {experts}")
+        if score == "softmax_all":
+            # scores: the softmax over all experts; the choice goes by score + correction, the weights by the scores
+            if correction is not None:
+                self._want(correction, "choice correction", torch.float32, (experts,))
+            self._check(self.core.sia_moe_route_corrected(_ptr(h), _ptr(router), _ptr(correction), _ptr(ids), _ptr(weights),
+                                                          n, width, experts, int(top), _DT[h.dtype], self._stream()),
+                        "moe_route")
+            return ids, weights
         self._check(self.core.sia_moe_route_ex(_ptr(h), _ptr(router), _ptr(ids), _ptr(weights), n, width, experts,
                                                int(top), _DT[h.dtype], int(score == "sigmoid"), count, keep, float(scale),
                                                self._stream()), "moe_route")
@@ -685,6 +765,68 @@ class HipKernels:
             _DT[proj.dtype], _ptr(workspace), self._stream()), "hgrn2_scan")
         return out
 
+    def delta_rule(self, qkv, proj, columns, a_log, dt_bias, norm_weight, n_heads, n_kv_heads, key_dim, value_dim, eps,
+                   ctx, state):
+        """The gated delta rule over the step's runs of tokens.  ``qkv`` rows are the convolved ``[q (kv_heads *
+        key_dim) | k (the same) | v (heads * value_dim)]``; ``columns = (g, b, a)`` name the output gates ``[heads *
+        value_dim]``, the write strengths' logits and the step sizes' inputs ``[heads]`` in the rows of ``proj``.  q
+        and k are made unit vectors per head (q also times ``key_dim ** -0.5``); ``beta = sigmoid(b)``, ``decay =
+        exp(-exp(a_log) * softplus(a + dt_bias))``; per head ``S <- decay S; S += k (beta (v - S^T k))^T; o = S^T q``;
+        ``o`` is divided by its root mean square, multiplied by ``norm_weight`` and by ``silu(g)``.  The matrices
+        ``[heads, key_dim, value_dim]`` are the first floats of a sequence's state row."""
+        self._want(qkv, "convolved rows")
+        self._want(proj, "projected rows", qkv.dtype)
+        n, width = qkv.shape
+        qk, inner = n_kv_heads * key_dim, n_heads * value_dim
+        if qkv.dtype not in _DT or n != ctx.n_tokens or proj.shape[0] != n or width != 2 * qk + inner:
+            raise KernelError(f"rows {qkv.dtype} {tuple(qkv.shape)} do not fit {ctx.n_tokens} tokens of {n_kv_heads} "
+                              f"query/key heads of {key_dim} and {n_heads} value heads of {value_dim}")
+        g, b, a = (int(c) for c in columns)
+        for first, size, what in ((g, inner, "gate"), (b, n_heads, "write strength"), (a, n_heads, "step size")):
+            if first < 0 or first + size > proj.shape[1]:
+                raise KernelError(f"columns {first} .. {first + size} of the {what} lie outside a row of {proj.shape[1]}")
+        for t, what in ((a_log, "decay rate"), (dt_bias, "step bias")):
+            self._want(t, what, torch.float32, (n_heads,))
+        self._want(norm_weight, "output norm weight", torch.float32, (value_dim,))
+        self.check_recurrent_geometry(key_dim, value_dim)
+        if n_kv_heads <= 0 or n_heads % n_kv_heads:
+            raise KernelError(f"{n_heads} value heads cannot share {n_kv_heads} query/key heads evenly")
+        stride = self._state_rows(state, ctx, n_heads * key_dim * value_dim)
+        out = torch.empty((n, inner), dtype=qkv.dtype, device=qkv.device)
+        workspace = self._float_workspace(ctx, self.core.sia_delta_rule_workspace(n, n_heads, value_dim), qkv.device)
+        self._check(self.core.sia_delta_rule(
+            _ptr(qkv), width, _ptr(proj), proj.shape[1], g, b, a, _ptr(a_log), _ptr(dt_bias), _ptr(norm_weight),
+            _ptr(state), stride, _ptr(ctx.cu_q), _ptr(ctx.state_slots), _ptr(out), n, ctx.n_seqs, ctx.max_q_len, n_heads,
+            n_kv_heads, key_dim, value_dim, float(eps), _DT[qkv.dtype], _ptr(workspace), self._stream()), "delta_rule")
+        return out
+
+    def decay_attention(self, proj, decays, norm_weight, n_heads, key_dim, value_dim, eps, ctx, state):
+        """Linear attention with a constant decay per head.  ``proj`` rows are ``[q | k (heads * key_dim each) | v | g
+        (heads * value_dim each)]`` and are used up (q, k and v are overwritten by their ``silu``).  Per head ``S <-
+        decays[h] S + k v^T``, ``o = S^T q``; the row of all heads' ``o`` is divided by its root mean square, multiplied
+        by ``norm_weight [heads * value_dim]`` and by ``sigmoid(g)``.  The state rows are ``[heads, key_dim,
+        value_dim]`` floats."""
+        self._want(proj, "projected rows")
+        n, width = proj.shape
+        qk, inner = n_heads * key_dim, n_heads * value_dim
+        if proj.dtype not in _DT or n != ctx.n_tokens or width != 2 * qk + 2 * inner:
+            raise KernelError(f"projected rows {proj.dtype} {tuple(proj.shape)} do not fit {ctx.n_tokens} tokens of "
+                              f"{n_heads} heads of {key_dim} and {value_dim}")
+        self._want(decays, "decays", torch.float32, (n_heads,))
+        self._want(norm_weight, "output norm weight", torch.float32, (inner,))
+        self.check_recurrent_geometry(key_dim, value_dim)
+        if state is None or tuple(state.shape[1:]) != (n_heads, key_dim, value_dim):
+            raise KernelError(f"state rows are not [{n_heads}, {key_dim}, {value_dim}]")
+        self._state_rows(state, ctx, qk * value_dim)
+        out = torch.empty((n, inner), dtype=proj.dtype, device=proj.device)
+        workspace = self._float_workspace(
+            ctx, self.core.sia_gla_workspace(n, ctx.n_seqs, ctx.max_q_len, n_heads, key_dim, value_dim), proj.device)
+        self._check(self.core.sia_decay_attention(
+            _ptr(proj), width, _ptr(decays), _ptr(norm_weight), _ptr(state), _ptr(ctx.cu_q), _ptr(ctx.state_slots),
+            _ptr(out), n, ctx.n_seqs, ctx.max_q_len, n_heads, key_dim, value_dim, float(eps), _DT[proj.dtype],
+            _ptr(workspace), self._stream()), "decay_attention")
+        return out
+
     # -- latent attention ---------------------------------------------------------------------
     def _rotation_tables(self, rotary_dim, cos, sin, ctx_or_len):
         if not rotary_dim:
@@ -756,10 +898,25 @@ class HipKernels:
             _ptr(positions) if rotary_dim else None, _DT[x.dtype], self._stream()), "headwise_linear")
         return y
 
-    def moe_experts(self, h, w_gate_up, w_down, ids, weights, shared=None, shared_gate=None):
+    @staticmethod
+    def _glu(activation):
+        """(kind, limit) of a gated activation as the kernels take it: None is ``silu(g) * u``, ``("clamped", limit)`` is
+        ``g * sigmoid(1.702 g) * (u + 1)`` with ``g = min(g, limit)`` and ``u = clamp(u, -limit, limit)``."""
+        if activation is None:
+            return _GLUS["silu"], 0.0
+        kind, limit = activation
+        if kind not in _GLUS or not float(limit) > 0:
+            raise KernelError(f"gated activation {activation!r} is not one of {', '.join(_GLUS)} with a positive limit")
+        return _GLUS[kind], float(limit)
+
+    def moe_experts(self, h, w_gate_up, w_down, ids, weights, shared=None, shared_gate=None, activation=None,
+                    identity=0):
         """``sum_k weights[n, k] * expert_{ids[n, k]}(h[n])`` with ``expert_e(x) = W2_e (silu(Wg_e x) * (Wu_e x))``,
         ``w_gate_up [E, 2 ff, width]`` (gate rows first), ``w_down [E, width, ff]``; plus ``shared`` ``[n, width]``
-        (times ``sigmoid(shared_gate [n, 1])`` if given), the sum rounded once."""
+        (times ``sigmoid(shared_gate [n, 1])`` if given), the sum rounded once.  ``activation``: another gated
+        activation than ``silu(g) * u`` (see ``_glu``); ``identity``: ids ``E .. E + identity - 1`` name experts
+        without tensors, which return their input."""
+        glu, limit = self._glu(activation)
         self._want(h, "expert input")
         n, width = h.shape
         experts, two_ff, _ = w_gate_up.shape
@@ -784,16 +941,16 @@ class HipKernels:
         if ints:
             workspace = torch.empty((ints,), dtype=torch.int32, device=h.device)
             y = torch.empty((n * top, width), dtype=h.dtype, device=h.device)
-            self._check(self.core.sia_moe_tiled(
+            self._check(self.core.sia_moe_tiled_ex(
                 _ptr(h), _ptr(w_gate_up), _ptr(w_down), _ptr(ids), _ptr(weights), _ptr(shared), _ptr(shared_gate),
-                gate_stride, _ptr(act), _ptr(y), _ptr(out), _ptr(workspace), n, width, ff, top, experts,
+                gate_stride, _ptr(act), _ptr(y), _ptr(out), _ptr(workspace), n, width, ff, top, experts, glu, limit,
                 self._stream()), "moe_tiled")
             return out
-        self._check(self.core.sia_moe_gate_up(_ptr(h), _ptr(w_gate_up), _ptr(ids), _ptr(act), n, width, ff, top,
-                                              _DT[h.dtype], self._stream()), "moe_gate_up")
-        self._check(self.core.sia_moe_down(_ptr(act), _ptr(w_down), _ptr(ids), _ptr(weights), _ptr(shared),
-                                           _ptr(shared_gate), gate_stride, _ptr(out), n, width, ff, top, _DT[h.dtype],
-                                           self._stream()), "moe_down")
+        self._check(self.core.sia_moe_gate_up_ex(_ptr(h), _ptr(w_gate_up), _ptr(ids), _ptr(act), n, width, ff, top,
+                                                 experts, glu, limit, _DT[h.dtype], self._stream()), "moe_gate_up")
+        self._check(self.core.sia_moe_down_ex(_ptr(act), _ptr(w_down), _ptr(ids), _ptr(weights), _ptr(shared),
+                                              _ptr(shared_gate), gate_stride, _ptr(out), n, width, ff, top, _ptr(h),
+                                              experts, _DT[h.dtype], self._stream()), "moe_down")
         return out
 
     # -- matrix product --------------------------------------------------------
@@ -835,11 +992,23 @@ class HipKernels:
             y = self.cast(y, back)
         return y
 
-    def gated_linear(self, x, w_gate_up):
-        """``silu(x Wg^T) * (x Wu^T)`` for ``w_gate_up = [Wg; Wu]``: one kernel for few rows, else product + SwiGLU."""
+    def gated_linear(self, x, w_gate_up, activation=None):
+        """``silu(x Wg^T) * (x Wu^T)`` for ``w_gate_up = [Wg; Wu]``: one kernel for few rows, else product + SwiGLU.
+        ``activation``: another gated activation (see ``_glu``), by the product and a kernel of its own."""
         self._want(w_gate_up, "gate/up weight")
         M, K = x.shape
         two_i = w_gate_up.shape[0]
+        if activation is not None:
+            glu, limit = self._glu(activation)
+            gu = self.linear(x, w_gate_up)
+            if gu.dtype not in _DT or two_i % 2:
+                raise KernelError(f"a gated activation takes [tokens, 2 * intermediate] rows, got {gu.dtype} {tuple(gu.shape)}")
+            out = torch.empty((M, two_i // 2), dtype=gu.dtype, device=gu.device)
+            for n0 in range(0, M, 65535):
+                n1 = min(M, n0 + 65535)
+                self._check(self.core.sia_glu(_ptr(gu[n0:n1]), _ptr(out[n0:n1]), n1 - n0, two_i // 2, glu, limit,
+                                              _DT[gu.dtype], self._stream()), "glu")
+            return out
         if (self.use_skinny_gemm and x.dtype == torch.bfloat16 and w_gate_up.dtype == torch.bfloat16
                 and M <= self._skinny_rows and two_i % 2 == 0 and K % 64 == 0 and w_gate_up.shape[1] == K):
             rows, partials, n_partials, eps = self._scaled(x)
@@ -1025,7 +1194,8 @@ class HipKernels:
             "rope_kv_write")
 
     def qkv_to_cache(self, x, w_qkv, n_heads, n_kv_written, head_dim, rotary_dim, cos, sin, ctx, cache,
-                     value_dim=None, bias=None, qk_norm=None, page_dim=None, q_temp=None, extra_columns=0):
+                     value_dim=None, bias=None, qk_norm=None, page_dim=None, q_temp=None, extra_columns=0,
+                     values_are_keys=False):
         """The q/k/v product, the rotation of q and k and the write of k and v into the pages.  Returns the
         ``[tokens, (n_heads + 2 n_kv_written) head_dim]`` matrix whose q columns hold the rotated queries; its
         k and v columns are not to be read (for few rows one kernel does all three and never writes them).
@@ -1040,10 +1210,12 @@ class HipKernels:
 
         ``q_temp``: ``(coef, every)``, every query is multiplied by ``1 + coef * ln(floor((pos + 1) / every) + 1)``
         after its norm.  ``extra_columns``: the weight has that many further rows behind v, whose products are only
-        carried along; the result is then the pair (that matrix, the further columns of the projected rows)."""
+        carried along; the result is then the pair (that matrix, the further columns of the projected rows).
+        ``values_are_keys``: the weight has no v rows; a position's values are its keys as projected (with their bias,
+        before norm and rotation)."""
         M, K = x.shape
         if (value_dim is not None or bias is not None or qk_norm is not None or page_dim is not None
-                or q_temp is not None or extra_columns):
+                or q_temp is not None or extra_columns or values_are_keys):
             qkv = self.linear(x, w_qkv)
             q_out = None
             if page_dim is not None:
@@ -1057,7 +1229,7 @@ class HipKernels:
                 if q_out is None:
                     q_out = kept[key] = torch.zeros((M, n_heads * page_dim), dtype=qkv.dtype, device=qkv.device)
             self.qk_prepare(qkv, n_heads, n_kv_written, head_dim, value_dim or head_dim, rotary_dim, cos, sin, bias,
-                            qk_norm, ctx, cache, page_dim, q_out, q_temp, extra_columns)
+                            qk_norm, ctx, cache, page_dim, q_out, q_temp, extra_columns, values_are_keys)
             queries = qkv if q_out is None else q_out
             if extra_columns:
                 return queries, qkv[:, qkv.shape[1] - extra_columns:]
@@ -1105,7 +1277,7 @@ class HipKernels:
         return wide
 
     def qk_prepare(self, qkv, n_heads, n_kv_written, head_dim, value_dim, rotary_dim, cos, sin, bias, qk_norm, ctx,
-                   cache, page_dim=None, q_out=None, q_temp=None, extra_columns=0):
+                   cache, page_dim=None, q_out=None, q_temp=None, extra_columns=0, values_are_keys=False):
         """Bias, per-head RMS norm of q and k, rotation, and the write of k and v into the pages, on the projected
         rows ``[q heads | k heads | v heads]`` (q and k heads ``head_dim`` wide, v heads ``value_dim``); q is left in
         place."""
@@ -1113,7 +1285,9 @@ class HipKernels:
         n, width = qkv.shape
         if qkv.dtype not in _DT:
             raise KernelError(f"qkv must be float32 or bfloat16, is {qkv.dtype}")
-        own = n_heads * head_dim + n_kv_written * (head_dim + value_dim)
+        if values_are_keys and (value_dim != head_dim or extra_columns):
+            raise KernelError("values that are the keys have the keys' width, and nothing rides behind them")
+        own = n_heads * head_dim + n_kv_written * (head_dim + (0 if values_are_keys else value_dim))
         if width != own + extra_columns:
             raise KernelError(f"qkv row of {width} does not hold {n_heads} q heads and {n_kv_written} k heads of "
                               f"{head_dim}, as many v heads of {value_dim} and {extra_columns} further columns")
@@ -1149,13 +1323,13 @@ class HipKernels:
         if n_kv_written:
             k_pages, v_pages, table, page_size = cache.k_pages, cache.v_pages, cache.block_table, cache.page_size
             self._check_pages(k_pages, v_pages, table, page_size, n_kv_written, k_row, qkv.dtype, ctx, v_rows)
-        self._check(self.core.sia_qk_prepare(
+        self._check(self.core.sia_qk_prepare_ex(
             _ptr(qkv), width, _ptr(bias), _ptr(q_gain), _ptr(k_gain), float(eps),
             _ptr(cos) if rotary_dim else None, _ptr(sin) if rotary_dim else None, _ptr(ctx.positions),
             _ptr(ctx.seq_of_token), _ptr(table), table.shape[1] if table is not None else 0, _ptr(k_pages),
             _ptr(v_pages), n, n_heads, n_kv_written, head_dim, value_dim, rotary_dim, page_size, k_row, v_rows,
-            _ptr(q_out), n_heads * page_dim if page_dim else 0, page_dim or 0, temp_coef, temp_every, _DT[qkv.dtype],
-            self._stream()), "qk_prepare")
+            _ptr(q_out), n_heads * page_dim if page_dim else 0, page_dim or 0, temp_coef, temp_every,
+            int(bool(values_are_keys)), _DT[qkv.dtype], self._stream()), "qk_prepare")
 
     def _check_pages(self, k_pages, v_pages, table, page_size, n_kv, head_dim, dtype, ctx, value_dim=None):
         value_dim = value_dim or head_dim

@@ -4,8 +4,8 @@ from .registry import (
     register_block, register_embedding, register_feed_forward, register_gate, register_head, register_mixer,
     register_norm, register_position_encoding, register_stream_op,
 )
-from .context import BiasedDelta, BuildEnv, LayerCache, ResidualStream, StepContext
-from . import norm, rope, attention, swiglu, dense, block, embedding, gate, stream_ops, gla, moe, ssm, hgrn, latent_attention  # noqa: F401  (registers the built-in kinds)
+from .context import BiasedDelta, BuildEnv, LayerCache, ResidualStream, ScaledSum, StepContext
+from . import norm, rope, attention, swiglu, dense, block, embedding, gate, stream_ops, gla, moe, ssm, hgrn, latent_attention, delta, decay_attention, parallel  # noqa: F401  (registers the built-in kinds)
 from .model import DecoderModel
 
 __all__ = [
@@ -13,5 +13,5 @@ __all__ = [
     "BLOCKS", "EMBEDDINGS", "FEED_FORWARDS", "GATES", "HEADS", "MIXERS", "NORMS", "POSITION_ENCODINGS", "STREAM_OPS",
     "register_block", "register_embedding", "register_feed_forward", "register_gate", "register_head", "register_mixer",
     "register_norm", "register_position_encoding", "register_stream_op",
-    "BiasedDelta", "BuildEnv", "LayerCache", "ResidualStream", "StepContext", "DecoderModel",
+    "BiasedDelta", "BuildEnv", "LayerCache", "ResidualStream", "ScaledSum", "StepContext", "DecoderModel",
 ]

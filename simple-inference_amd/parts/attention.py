@@ -32,6 +32,8 @@ Further forms, each switched on by a parameter of its own and free to combine:
   ``1 + c * ln(floor((p + 1) / n) + 1)`` after its norm, so late queries score more sharply.
 * ``out_gate``: head ``h``'s output is multiplied by ``sigmoid((G x)_h)``, a scalar for every token and head, ``G
   [Hq, H]`` reading the mixer's own input; its rows ride at the end of the stacked projection.
+* ``value_from_key``: there is no value projection: a position's values are its keys as projected (with their bias,
+  before norm and rotation); the stacked matrix is ``[(Hq + Hkv) D, H]``.
 * ``o_bias``: the output projection has a bias; it is handed on with the result (``BiasedDelta``) so that the sum
   into the residual can take it in passing.
 """
@@ -58,7 +60,7 @@ def _shared_position_encoding(spec, env):
 class Attention:
     """params: hidden_size, num_heads, num_kv_heads, head_dim, position
     (``{"kind", "params"}``), and optionally window, scale, kv_from_layer, value_head_dim, bias, qk_norm, chunk,
-    sink, q_temp, out_gate, o_bias."""
+    sink, q_temp, out_gate, o_bias, value_from_key."""
 
     def __init__(self, params, env):
         self.hidden = int(params["hidden_size"])
@@ -86,6 +88,9 @@ class Attention:
             raise ValueError(f"q_temp.every must be positive, got {self.q_temp[1]}")
         self.out_gate = bool(params.get("out_gate", False))
         self.o_bias = bool(params.get("o_bias", False))
+        self.value_from_key = bool(params.get("value_from_key", False))
+        if self.value_from_key and (self.value_dim != self.head_dim or params.get("kv_from_layer") is not None):
+            raise ValueError("values that are the keys have the keys' width, and the mixer projects its own keys")
         self.chunk = params.get("chunk")
         if self.chunk is not None:
             self.chunk = int(self.chunk)
@@ -123,10 +128,12 @@ class Attention:
         specs = {"q": TensorSpec((q, self.hidden)), "o": TensorSpec((self.hidden, self.num_heads * self.value_dim))}
         if self.writes_kv:
             specs["k"] = TensorSpec((kv, self.hidden))
-            specs["v"] = TensorSpec((v, self.hidden))
+            if not self.value_from_key:
+                specs["v"] = TensorSpec((v, self.hidden))
         if self.bias:
-            specs.update({"q_bias": TensorSpec((q,), "vector"), "k_bias": TensorSpec((kv,), "vector"),
-                          "v_bias": TensorSpec((v,), "vector")})
+            specs.update({"q_bias": TensorSpec((q,), "vector"), "k_bias": TensorSpec((kv,), "vector")})
+            if not self.value_from_key:
+                specs["v_bias"] = TensorSpec((v,), "vector")
         if self.qk_norm_eps is not None and self.qk_norm_gain:
             specs.update({"q_norm": TensorSpec((self.head_dim,), "vector"), "k_norm": TensorSpec((self.head_dim,), "vector")})
         if self.sink:
@@ -138,7 +145,9 @@ class Attention:
         return specs
 
     def bind(self, tensors):
-        stacked = [tensors["q"], tensors["k"], tensors["v"]] if self.writes_kv else [tensors["q"]]
+        stacked = [tensors["q"]]
+        if self.writes_kv:
+            stacked += [tensors["k"]] if self.value_from_key else [tensors["k"], tensors["v"]]
         if self.out_gate:   # the gate's rows behind v, filled up with zero rows so that a projected row stays aligned
             self.gate_columns = -(-self.num_heads // 8) * 8
             g = tensors["gate"]
@@ -150,7 +159,7 @@ class Attention:
             wide[:, :, :self.value_dim] = self.w_o.view(self.hidden, self.num_heads, self.value_dim)
             self.w_o = wide.view(self.hidden, self.num_heads * self.page_dim)
         if self.bias:
-            self.b_qkv = torch.cat([tensors["q_bias"], tensors["k_bias"], tensors["v_bias"]]).contiguous()
+            self.b_qkv = torch.cat([tensors[n] for n in ("q_bias", "k_bias", "v_bias") if n in tensors]).contiguous()
         if self.qk_norm_eps is not None and self.qk_norm_gain:
             self.q_gain, self.k_gain = tensors["q_norm"].contiguous(), tensors["k_norm"].contiguous()
         elif self.qk_norm_eps is not None:
@@ -177,7 +186,7 @@ class Attention:
     def _options(self) -> bool:
         """Whether any of the further forms is switched on (the kernels then get them as keyword arguments)."""
         return (self.bias or self.qk_norm_eps is not None or self.sink or self.chunk is not None
-                or self.value_dim != self.head_dim or self.q_temp is not None or self.out_gate)
+                or self.value_dim != self.head_dim or self.q_temp is not None or self.out_gate or self.value_from_key)
 
     def cache_need(self):
         if self.page_dim is not None:
@@ -211,6 +220,8 @@ class Attention:
                 project["q_temp"] = self.q_temp
             if self.out_gate:
                 project["extra_columns"] = self.gate_columns
+            if self.value_from_key:
+                project["values_are_keys"] = True
         qkv = k.qkv_to_cache(
             h, self.w_qkv, self.num_heads, self.num_kv_heads if self.writes_kv else 0, self.head_dim,
             self.position.rotary_dim, cos, sin, ctx, cache, **project)

@@ -3,7 +3,9 @@
 Pre-norm (reference: ``model/block.py:135-147``):
 ``x += mixer(norm1(x))``; ``x += feed_forward(norm2(x))``.  Each add is carried
 as the stream's pending delta and summed into the float32 residual by the norm
-that follows (the next layer's, or the model's last norm).
+that follows (the next layer's, or the model's last norm).  With ``residual_scale`` (a parameter of the block, from
+the layer's ``block_params``) every sublayer's result is multiplied by that constant on its way into the residual
+(``stream.scale``); a pre-norm layer may have no feed-forward.
 
 Output-norm: ``x += norm1(mixer(x))``; ``x += norm2(feed_forward(x))``.  Mixer and feed-forward take the
 un-normed stream as input (rounded to the compute dtype), and each norm is applied to its sublayer's result; the kernel that adds the normed
@@ -23,18 +25,21 @@ from .registry import register_block
 
 @register_block("prenorm")
 class PreNormBlock:
-    def __init__(self, mixer, feed_forward, mixer_norm, feed_forward_norm):
+    def __init__(self, mixer, feed_forward=None, mixer_norm=None, feed_forward_norm=None, residual_scale=None):
+        if mixer_norm is None or (feed_forward is None) != (feed_forward_norm is None):
+            raise ValueError("a pre-norm block has a mixer with its norm, and a feed-forward with its norm or neither")
         self.mixer = mixer
         self.feed_forward = feed_forward
         self.mixer_norm = mixer_norm
         self.feed_forward_norm = feed_forward_norm
+        self.residual_scale = None if residual_scale is None or float(residual_scale) == 1.0 else float(residual_scale)
         self.plain_forms = None   # kept by kernels that run the block in one call: what they made of the parts
 
     def plain_form(self):
         """What this block is, as plain data, for kernels that can make all of its launches in one call: its kind
         (the order in which the parts run is this file's affair: the docstring above) and what each part says it is
         (its own ``plain_form``; None for a part that has none, and such a block goes part by part)."""
-        if type(self).forward is not PreNormBlock.forward:
+        if type(self).forward is not PreNormBlock.forward or self.residual_scale is not None or self.feed_forward is None:
             return None
         form = lambda part: getattr(part, "plain_form", lambda: None)()
         return {"kind": "prenorm", "mixer_norm": form(self.mixer_norm), "mixer": form(self.mixer),
@@ -48,8 +53,12 @@ class PreNormBlock:
             return
         h = _normed(self.mixer_norm, self.mixer, stream)
         stream.delta = self.mixer.forward(h, ctx, cache)
+        stream.scale = self.residual_scale
+        if self.feed_forward is None:
+            return
         h = _normed(self.feed_forward_norm, self.feed_forward, stream)
         stream.delta = self.feed_forward.forward(h, ctx)
+        stream.scale = self.residual_scale
 
 
 def _normed(norm, consumer, stream):

@@ -84,9 +84,13 @@ class ResidualStream:
     (``residual += post(delta)``, for blocks that norm a sublayer's result as well as its input).  It is set after
     the delta and forgotten with it; a norm that can apply it inside its own kernel does so, everybody else has it
     applied by ``settle`` (the norm's ``add_normed``).
+
+    ``scale`` belongs to the pending delta as well: a constant factor on its way into the residual (``residual +=
+    scale * delta``), set after the delta and forgotten with it.  A delta may be a ``ScaledSum``, several results
+    with a factor each that nobody has added up yet; a sum that can take the terms one by one does.
     """
 
-    __slots__ = ("residual", "raw_delta", "lowered", "gate", "post")
+    __slots__ = ("residual", "raw_delta", "lowered", "gate", "post", "scale")
 
     def __init__(self, residual: torch.Tensor, delta: Optional[torch.Tensor] = None):
         self.residual = residual
@@ -94,6 +98,7 @@ class ResidualStream:
         self.lowered = None
         self.gate = None
         self.post = None
+        self.scale = None
 
     @property
     def delta(self):
@@ -106,13 +111,27 @@ class ResidualStream:
         self.raw_delta = value
         self.gate = None
         self.post = None
+        self.scale = None
         if value is not None:
             self.lowered = None
+
+    def scaled_terms(self):
+        """The pending delta as ``[(tensor, factor)]`` with the stream's own factor multiplied in."""
+        raw, own = self.raw_delta, 1.0 if self.scale is None else float(self.scale)
+        if isinstance(raw, ScaledSum):
+            return [(y, f * own) for y, f in raw.values()]
+        return [(self.delta, own)]
 
     def settle(self, kernels) -> torch.Tensor:
         """Adds what is pending into the residual (no norm follows) and returns the residual."""
         raw = self.raw_delta
         if raw is None:
+            return self.residual
+        if self.scale is not None or isinstance(raw, ScaledSum):
+            if self.post is not None or self.gate is not None:
+                raise NotImplementedError("a scaled delta passes neither a gate nor a norm of its own")
+            kernels.add_rmsnorm(self.residual, None, None, 0.0, self.residual.dtype, terms=self.scaled_terms())
+            self.delta = None
             return self.residual
         if self.post is not None:
             post = self.post
@@ -128,6 +147,25 @@ class ResidualStream:
         kernels.gated_add(self.residual, raw, gate, gate_bias, bias)
         self.delta = None
         return self.residual
+
+
+class ScaledSum:
+    """A sublayer's result that is a sum of several, each with a constant factor: ``sum_i factor_i * y_i``.  A sum
+    into the residual that can take the terms one by one reads ``terms``; everybody else gets the tensor from
+    ``compute()``."""
+
+    __slots__ = ("terms", "kernels")
+
+    def __init__(self, terms, kernels):
+        self.terms, self.kernels = list(terms), kernels
+
+    def values(self):
+        """``[(tensor, factor)]``, products that were left pending computed."""
+        self.terms = [(y.compute() if hasattr(y, "compute") else y, f) for y, f in self.terms]
+        return self.terms
+
+    def compute(self):
+        return self.kernels.scaled_sum(self.values())
 
 
 class BiasedDelta:

@@ -1,7 +1,7 @@
 """Dense feed-forward without a gate: ``y = act(h Wu^T) Wd^T``.
 
 ``act`` is named by the ``activation`` parameter: ``relu2`` is the square of ``max(z, 0)``, ``gelu_tanh`` is
-``0.5 z (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3)))``.  The activation is computed in float32 on the product and
+``0.5 z (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3)))``, ``gelu`` is ``0.5 z (1 + erf(z / sqrt(2)))``.  The activation is computed in float32 on the product and
 rounded once; for few rows it is part of the product's own kernel.
 """
 
@@ -10,7 +10,7 @@ from __future__ import annotations
 from .plan import TensorSpec
 from .registry import register_feed_forward
 
-ACTIVATIONS = ("relu2", "gelu_tanh")
+ACTIVATIONS = ("relu2", "gelu_tanh", "gelu")
 
 
 @register_feed_forward("dense")

@@ -46,9 +46,10 @@ class _Layer:
         self.named = {name: _REGISTRY_OF_ROLE[ps.role].get(ps.kind)(ps.params, env) for name, ps in spec.parts.items()}
         block_cls = BLOCKS.get(spec.block)
         try:
-            self.block = block_cls(**self.named)
+            self.block = block_cls(**self.named, **spec.block_params)
         except TypeError as exc:
-            raise ValueError(f"a {spec.block!r} block does not take the parts {sorted(self.named)}: {exc}") from None
+            raise ValueError(f"a {spec.block!r} block does not take the parts {sorted(self.named)}"
+                             f"{' with ' + str(sorted(spec.block_params)) if spec.block_params else ''}: {exc}") from None
         self.mixer = next((self.named[name] for name, ps in spec.parts.items() if ps.role == "mixer"), None)
         self.parts = [(self.named[name], ps) for name, ps in spec.parts.items()]
 

@@ -10,16 +10,20 @@ the norm of what the sublayer returned, ``x += y * rsqrt(mean(y^2) + eps) * w``,
 
 from __future__ import annotations
 
-from .context import BiasedDelta
+from .context import BiasedDelta, ScaledSum
 from .plan import TensorSpec
 from .registry import register_norm
 
 
 @register_norm("rmsnorm")
 class RMSNorm:
+    """params: size, eps, and optionally unit_offset (default False): the stored vector is the gain's distance from
+    one, ``y = x * rsqrt(mean(x^2) + eps) * (1 + w)``; the one is added once, in float32, when the vector is bound."""
+
     def __init__(self, params, env):
         self.size = int(params["size"])
         self.eps = float(params["eps"])
+        self.unit_offset = bool(params.get("unit_offset", False))
         self.env = env
         self.weight = None
 
@@ -28,6 +32,8 @@ class RMSNorm:
 
     def bind(self, tensors):
         self.weight = tensors["weight"]
+        if self.unit_offset:
+            self.weight = (self.weight.float() + 1.0).contiguous()
 
     gives_scaled_rows = True
 
@@ -36,6 +42,7 @@ class RMSNorm:
         subclass with a forward of its own: it is no longer what this form describes)."""
         if type(self).forward is not RMSNorm.forward:
             return None
+        # (a gain stored as its distance from one is an ordinary gain once it is bound)
         return {"kind": "rmsnorm", "weight": self.weight, "eps": self.eps, "size": self.size}
 
     def add_normed(self, stream, y):
@@ -62,6 +69,13 @@ class RMSNorm:
             stream.settle(k)
         if stream.gate is not None or isinstance(stream.raw_delta, BiasedDelta):
             return self._gated(stream, rows)
+        if stream.scale is not None or isinstance(stream.raw_delta, ScaledSum):
+            # the delta, or its several terms, with a constant factor each: all added inside the norm's kernel
+            out = k.add_rmsnorm(stream.residual, None, self.weight, self.eps, self.env.dtype, rows,
+                                terms=stream.scaled_terms())
+            if rows is None:
+                stream.delta = None
+            return out
         if scaled_ok and rows is None and hasattr(stream.raw_delta, "compute") and hasattr(k, "linear_into_residual"):
             out = k.linear_into_residual(stream.raw_delta, stream.residual, self.weight, self.eps)
             stream.delta = None

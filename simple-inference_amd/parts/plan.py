@@ -53,6 +53,7 @@ class LayerSpec:
     feed_forward_norm: Optional[PartSpec] = None
     block: str = "prenorm"
     parts: Dict[str, PartSpec] = field(default_factory=dict)
+    block_params: Dict[str, Any] = field(default_factory=dict)   # constants of the block kind itself, by keyword
 
     def __post_init__(self):
         short = (("mixer_norm", "norm"), ("mixer", "mixer"), ("feed_forward_norm", "norm"), ("feed_forward", "feed_forward"))

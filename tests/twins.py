@@ -36,8 +36,12 @@ class TwinKernels:
 
     # -- residual add + rms norm ---------------------------------------------
     def add_rmsnorm(self, residual, delta, weight, eps, out_dtype, rows=None, gate=None, gate_bias=None,
-                    delta_bias=None):
-        if delta is not None:
+                    delta_bias=None, terms=None):
+        if terms is not None:      # the delta as several results with a constant factor each
+            delta = None
+            for y, f in terms:
+                delta = y.float() * f if delta is None else delta + y.float() * f
+        elif delta is not None:
             delta = self._gated(delta, gate, gate_bias, delta_bias)
         if rows is None:
             if delta is not None:
@@ -47,8 +51,16 @@ class TwinKernels:
             x = residual[rows.long()]
             if delta is not None:
                 x = x + delta[rows.long()]
+        if weight is None:
+            return None
         var = x.pow(2).mean(-1, keepdim=True)
         return (x * torch.rsqrt(var + eps) * weight.float()).to(out_dtype)
+
+    def scaled_sum(self, terms):
+        total = None
+        for y, f in terms:
+            total = y.float() * f if total is None else total + y.float() * f
+        return total.to(terms[0][0].dtype)
 
     @staticmethod
     def _gated(delta, gate, gate_bias, delta_bias):
@@ -141,7 +153,7 @@ class TwinKernels:
             past = state[slots[s], state_offset:state_offset + channels * (taps - 1)].view(taps - 1, channels)
             seq = torch.cat([past, u[cu[s]:cu[s + 1]]], dim=0)
             n = cu[s + 1] - cu[s]
-            acc = bias.float().expand(n, channels).clone()
+            acc = bias.float().expand(n, channels).clone() if bias is not None else torch.zeros(n, channels)
             for j in range(taps):
                 acc += seq[j:j + n] * w[:, j]
             out[cu[s]:cu[s + 1]] = acc
@@ -172,6 +184,50 @@ class TwinKernels:
         parts = y.view(n, norm_groups, inner // norm_groups)
         y = (parts * torch.rsqrt(parts.pow(2).mean(-1, keepdim=True) + eps)).view(n, inner) * norm_weight.float()
         return y.to(proj.dtype)
+
+    def delta_rule(self, qkv, proj, columns, a_log, dt_bias, norm_weight, n_heads, n_kv_heads, key_dim, value_dim, eps,
+                   ctx, state):
+        n, H, G, D, Dv = qkv.shape[0], n_heads, n_kv_heads, key_dim, value_dim
+        cg, cb, ca = columns
+        x, p = qkv.float(), proj.float()
+        q = x[:, :G * D].view(n, G, D)
+        k = x[:, G * D:2 * G * D].view(n, G, D)
+        v = x[:, 2 * G * D:].view(n, H, Dv)
+        q = q * torch.rsqrt(q.pow(2).sum(-1, keepdim=True) + 1e-6) * D ** -0.5
+        k = k * torch.rsqrt(k.pow(2).sum(-1, keepdim=True) + 1e-6)
+        q, k = q.repeat_interleave(H // G, dim=1), k.repeat_interleave(H // G, dim=1)
+        beta = torch.sigmoid(p[:, cb:cb + H])
+        step = torch.nn.functional.softplus(p[:, ca:ca + H] + dt_bias.float(), threshold=1e9)
+        decay = torch.exp(-torch.exp(a_log.float()) * step)
+        out = torch.zeros(n, H, Dv)
+        cu, slots = ctx.cu_q.tolist(), ctx.state_slots.tolist()
+        for s in range(ctx.n_seqs):
+            S = state[slots[s], :H * D * Dv].view(H, D, Dv)
+            for t in range(cu[s], cu[s + 1]):
+                S.mul_(decay[t][:, None, None])
+                u = beta[t][:, None] * (v[t] - torch.einsum("hd,hdv->hv", k[t], S))
+                S.add_(k[t][:, :, None] * u[:, None, :])
+                out[t] = torch.einsum("hd,hdv->hv", q[t], S)
+        out = out * torch.rsqrt(out.pow(2).mean(-1, keepdim=True) + eps) * norm_weight.float()
+        return (out.view(n, H * Dv) * torch.nn.functional.silu(p[:, cg:cg + H * Dv])).to(qkv.dtype)
+
+    def decay_attention(self, proj, decays, norm_weight, n_heads, key_dim, value_dim, eps, ctx, state):
+        n, H, D, Dv = proj.shape[0], n_heads, key_dim, value_dim
+        act = torch.nn.functional.silu(proj[:, :2 * H * D + H * Dv].float()).to(proj.dtype).float()
+        q = act[:, :H * D].view(n, H, D)
+        k = act[:, H * D:2 * H * D].view(n, H, D)
+        v = act[:, 2 * H * D:].view(n, H, Dv)
+        g = proj[:, 2 * H * D + H * Dv:].float()
+        out = torch.zeros(n, H, Dv)
+        cu, slots = ctx.cu_q.tolist(), ctx.state_slots.tolist()
+        for s in range(ctx.n_seqs):
+            S = state[slots[s]]
+            for t in range(cu[s], cu[s + 1]):
+                S.mul_(decays.float()[:, None, None]).add_(k[t][:, :, None] * v[t][:, None, :])
+                out[t] = torch.einsum("hd,hdv->hv", q[t], S)
+        out = out.view(n, H * Dv)
+        out = out * torch.rsqrt(out.pow(2).mean(-1, keepdim=True) + eps) * norm_weight.float()
+        return (out * torch.sigmoid(g)).to(proj.dtype)
 
     def hgrn2_scan(self, proj, f_bias, lower, norm_weight, n_heads, key_dim, value_dim, eps, ctx, state):
         n, H, D, Dv = proj.shape[0], n_heads, key_dim, value_dim
@@ -238,8 +294,14 @@ class TwinKernels:
         return y.view(n, H * out_stride).to(x.dtype)
 
     # -- mixture of experts ---------------------------------------------------------
-    def moe_route(self, h, router, top, score="softmax", groups=None, scale=1.0):
+    def moe_route(self, h, router, top, score="softmax", groups=None, scale=1.0, correction=None):
         logits = h.float() @ router.float().T
+        if score == "softmax_all":
+            sc = torch.softmax(logits, -1)
+            ranked = sc + correction.float() if correction is not None else sc
+            order = torch.sort(ranked, dim=-1, descending=True, stable=True).indices[:, :top]
+            chosen = torch.gather(sc, 1, order)
+            return order.to(torch.int32), chosen / (chosen.sum(-1, keepdim=True) + 1e-20)
         if score == "sigmoid":
             sc = torch.sigmoid(logits)
             ranked = sc
@@ -258,16 +320,31 @@ class TwinKernels:
         best = torch.gather(logits, 1, order)
         return order.to(torch.int32), torch.softmax(best, -1)
 
-    def moe_experts(self, h, w_gate_up, w_down, ids, weights, shared=None, shared_gate=None):
+    @staticmethod
+    def _glu(g, u, activation):
+        if activation is None:
+            return torch.nn.functional.silu(g) * u
+        kind, limit = activation
+        assert kind == "clamped"
+        g, u = g.clamp(max=limit), u.clamp(-limit, limit)
+        return g * torch.sigmoid(1.702 * g) * (u + 1.0)
+
+    def moe_experts(self, h, w_gate_up, w_down, ids, weights, shared=None, shared_gate=None, activation=None,
+                    identity=0):
         n, top = ids.shape
         ff = w_gate_up.shape[1] // 2
+        real = w_gate_up.shape[0]
         x = h.float()
         y = torch.zeros(n, w_down.shape[1])
         for t in range(n):
             for k in range(top):
                 e = int(ids[t, k])
+                if e >= real:       # an expert without tensors: its input comes back
+                    assert e < real + identity
+                    y[t] += weights[t, k] * x[t]
+                    continue
                 gu = w_gate_up[e].float() @ x[t]
-                a = (torch.nn.functional.silu(gu[:ff]) * gu[ff:]).to(h.dtype).float()
+                a = self._glu(gu[:ff], gu[ff:], activation).to(h.dtype).float()
                 y[t] += weights[t, k] * (w_down[e].float() @ a)
         if shared is not None:
             s = shared.float()
@@ -283,7 +360,11 @@ class TwinKernels:
 
     pending_linear = linear   # computed at once: the twin's norm always has a kernel of its own
 
-    def gated_linear(self, x, w_gate_up):
+    def gated_linear(self, x, w_gate_up, activation=None):
+        if activation is not None:
+            gu = self.linear(x, w_gate_up).float()
+            inter = gu.shape[-1] // 2
+            return self._glu(gu[:, :inter], gu[:, inter:], activation).to(x.dtype)
         return self.swiglu(self.linear(x, w_gate_up))
 
     # -- feed-forward activation --------------------------------------------
@@ -298,22 +379,25 @@ class TwinKernels:
             a = torch.relu(z) ** 2
         elif activation == "gelu_tanh":
             a = 0.5 * z * (1 + torch.tanh(0.7978845608028654 * (z + 0.044715 * z ** 3)))
+        elif activation == "gelu":
+            a = 0.5 * z * (1 + torch.erf(z * 0.7071067811865476))
         else:
             raise ValueError(activation)
         return a.to(x.dtype)
 
     def qkv_to_cache(self, x, w_qkv, n_heads, n_kv_written, head_dim, rotary_dim, cos, sin, ctx, cache,
-                     value_dim=None, bias=None, qk_norm=None, q_temp=None, extra_columns=0):
+                     value_dim=None, bias=None, qk_norm=None, q_temp=None, extra_columns=0, values_are_keys=False):
         qkv = self.linear(x, w_qkv)
         self.rope_kv_write(qkv, n_heads, n_kv_written, head_dim, rotary_dim, cos, sin, ctx, cache,
-                           value_dim=value_dim, bias=bias, qk_norm=qk_norm, q_temp=q_temp)
+                           value_dim=value_dim, bias=bias, qk_norm=qk_norm, q_temp=q_temp,
+                           values_are_keys=values_are_keys)
         if extra_columns:
             return qkv, qkv[:, qkv.shape[1] - extra_columns:]
         return qkv
 
     # -- rotation + cache write ----------------------------------------------
     def rope_kv_write(self, qkv, n_heads, n_kv_written, head_dim, rotary_dim, cos, sin, ctx, cache,
-                      value_dim=None, bias=None, qk_norm=None, q_temp=None):
+                      value_dim=None, bias=None, qk_norm=None, q_temp=None, values_are_keys=False):
         N = qkv.shape[0]
         pos = ctx.positions.long()
         value_dim = value_dim or head_dim
@@ -350,7 +434,7 @@ class TwinKernels:
             return
         kv0 = n_heads * head_dim
         k = qkv[:, kv0:kv0 + n_kv_written * head_dim].view(N, n_kv_written, head_dim)
-        v0 = kv0 + n_kv_written * head_dim
+        v0 = kv0 if values_are_keys else kv0 + n_kv_written * head_dim      # the keys as projected serve as values
         v = qkv[:, v0:v0 + n_kv_written * value_dim].view(N, n_kv_written, value_dim)
         k = rotate(normed(k, qk_norm[1] if qk_norm else None))
         ps = cache.page_size
