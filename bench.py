@@ -29,6 +29,8 @@ feed-forwards and a model of linear-attention layers with routed experts, each b
 ``--workload famepel`` does the same for the Famepel design: a model of each of its three mixers (state-space,
 forget-gate recurrence, latent attention), all with grouped experts, beside the Mogisun model of linear-attention
 layers with routed experts and the Llama model.
+``--workload tadinex`` does the same for the Tadinex design: a model of delta-rule layers and a model of layers with a
+windowed attention beside a decaying linear attention, both with clamped experts, beside the same two models.
 
 The engine runs on one GPU; asked for more it says so and exits with 2.
 """
@@ -81,11 +83,11 @@ def parse_args(argv=None):
     ap.add_argument("--temperature", type=float, default=0.0, help="sampling of the decode measurement (0: greedy)")
     ap.add_argument("--top-k", type=int, default=0)
     ap.add_argument("--top-p", type=float, default=1.0)
-    ap.add_argument("--workload", default="decode", choices=["decode", "continuous", "shared-prefix", "feduzen", "mogisun", "famepel"])
+    ap.add_argument("--workload", default="decode", choices=["decode", "continuous", "shared-prefix", "feduzen", "mogisun", "famepel", "tadinex"])
     ap.add_argument("--shapes", default="1b,3b,8b", help="--workload feduzen: which layer sizes, comma separated")
-    ap.add_argument("--models", default=None, help="--workload feduzen, mogisun or famepel: which of the models to run "
+    ap.add_argument("--models", default=None, help="--workload feduzen, mogisun, famepel or tadinex: which of the models to run "
                     "(feduzen,llama; mogisun-attention,mogisun-linear,llama; famepel-ssm,famepel-hgrn,famepel-latent,"
-                    "mogisun-linear,llama)")
+                    "mogisun-linear,llama; tadinex-delta,tadinex-parallel,mogisun-linear,llama)")
     ap.add_argument("--max-running", type=int, default=64, help="request slots of the stream workloads")
     return ap.parse_args(argv)
 
@@ -533,6 +535,61 @@ def famepel_workload(args):
     return 0
 
 
+def tadinex_config_like(llama_cfg, layers, kind):
+    """A Tadinex config.json with the width, head count, head width and feed-forward size of a Llama one; every layer
+    has the same mixer and eight experts of a quarter of the feed-forward size beside two identity experts, two a
+    token, and a shared expert of half of it (as many active feed-forward weights as the dense layer has, as the
+    Mogisun model beside it).  ``delta``: as many value heads of the head width, the Llama model's number of
+    key/value heads as query/key heads, a convolution of four taps.  ``parallel``: the Llama model's attention heads
+    with a window wider than the measured context (so that both models' attention does equal work), a rotation of
+    half of every head with ramp-scaled frequencies, beside a decaying linear attention with as many heads as the
+    Llama model has key/value heads."""
+    dim, heads, width = llama_cfg["head_dim"], llama_cfg["num_attention_heads"], llama_cfg["hidden_size"]
+    kv, ff = llama_cfg["num_key_value_heads"], llama_cfg["intermediate_size"]
+    if kind == "delta":
+        mixer = {"type": "delta", "mixer": {"conv": 4, "dim": dim, "heads": heads, "kv_heads": kv, "vdim": dim}}
+    else:
+        mixer = {"type": "parallel", "mixer": {
+            "left": {"dim": dim, "vdim": dim, "heads": heads, "kv_heads": kv, "mask": {"size": 1 << 20}, "scale": dim ** -0.5,
+                     "rot": {"base": llama_cfg["rope_theta"], "dims": dim // 2,
+                             "scaling": {"factor": 8.0, "original": 8192, "fast": 32.0, "slow": 1.0}}},
+            "left_scale": 0.7,
+            "right": {"dim": dim, "vdim": dim, "heads": kv, "decay": [1.0 - 2.0 ** -(3 + i % 6) for i in range(kv)]},
+            "right_scale": 0.9}}
+    mlp = {"kind": "moe", "expert": {"ff": ff // 4, "limit": 7.0}, "router": {"experts": 8, "identity": 2, "top": 2},
+           "shared": {"ff": ff // 2, "limit": 7.0}}
+    return {"architecture": "Tadinex", "vocab": llama_cfg["vocab_size"], "width": width,
+            "norm": {"eps": llama_cfg["rms_norm_eps"]}, "embedding": {"scale": 1.0}, "residual_mult": 0.5,
+            "layers": [json.loads(json.dumps(dict(mixer, mlp=mlp))) for _ in range(layers)]}
+
+
+def tadinex_workload(args):
+    """Decode and prefill of the Tadinex design (each of its two mixers alone, with its experts) beside the Mogisun
+    model of linear-attention layers with routed experts and the Llama model at equal layer sizes."""
+    layers = args.layers or 8
+    dt_name = "bf16" if args.dtype == "bfloat16" else "fp32"
+    out = measure_beside(args, lambda llama, n: (("tadinex-delta", tadinex_config_like(llama, n, "delta")),
+                                                 ("tadinex-parallel", tadinex_config_like(llama, n, "parallel")),
+                                                 ("mogisun-linear", mogisun_config_like(llama, n, "linear")),
+                                                 ("llama", llama)),
+                         (args.models or "tadinex-delta,tadinex-parallel,mogisun-linear,llama").split(","))
+    line = {"metric": "Tadinex beside Mogisun and Llama at equal layer sizes: decode tok/s (batch 8, 1) and prefill tok/s",
+            "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "dtype": dt_name,
+            "data": "synthetic (seeded random weights and uniform-random token ids)",
+            "config": {"layers": layers, "context": args.context, "prefill_tokens": args.prefill_tokens,
+                       "shapes": FEDUZEN_SHAPES,
+                       "tadinex-*": "scaled pre-norm sublayers; 8 clamped experts of ff/4 and 2 identity experts, 2 a "
+                                    "token, a shared expert of ff/2",
+                       "tadinex-delta": "gated delta rule: value heads of the head width, the Llama model's key/value "
+                                        "heads as query/key heads, 4 taps",
+                       "tadinex-parallel": "the Llama model's attention heads (window beyond the context, q/k norm, "
+                                           "sinks, values that are the keys) beside a decaying linear attention",
+                       "mogisun-linear": "gated linear attention, 8 experts of ff/4 (2 a token) and a shared one of ff/2"},
+            "shapes": out}
+    print(json.dumps(line), flush=True)
+    return 0
+
+
 def further_points(args, pts, config, layer_w, head_w, el):
     """What the headline leaves out, at sizes a server meets: the same model with contexts of 8,192 and 32,768 tokens
     and a prompt of 8,192 (an engine of its own with a context limit of 33,792), and the two request streams of the
@@ -605,6 +662,8 @@ def main(argv=None):
         return mogisun_workload(args)
     if args.workload == "famepel":
         return famepel_workload(args)
+    if args.workload == "tadinex":
+        return tadinex_workload(args)
     if args.workload != "decode":
         return stream_workload(args)
     points = [int(p) for p in args.points.split(",") if p]
