@@ -36,6 +36,22 @@ def _famepel_layer(mixer):
                             "router": {"experts": 8, "top": 2, "scale": 2.0, "groups": {"count": 4, "keep": 2}}})
 
 
+def _tadinex_layer(kind, mlp):
+    if kind == "delta":
+        mixer = {"conv": 4, "dim": 64, "heads": 8, "kv_heads": 4, "vdim": 64}
+    else:
+        mixer = {"left": {"dim": 64, "vdim": 64, "heads": 8, "kv_heads": 2, "mask": {"size": 128}, "scale": 0.125,
+                          "rot": {"base": 100000.0, "dims": 32,
+                                  "scaling": {"factor": 4.0, "original": 1024, "fast": 32.0, "slow": 1.0}}},
+                 "left_scale": 0.7, "right": {"dim": 64, "vdim": 64, "heads": 4, "decay": [0.75, 0.9, 0.97, 0.995]},
+                 "right_scale": 0.9}
+    return {"type": kind, "mixer": mixer, "mlp": mlp}
+
+
+_TADINEX_EXPERTS = {"kind": "moe", "router": {"experts": 8, "identity": 2, "top": 2}, "expert": {"ff": 256, "limit": 7.0},
+                    "shared": {"ff": 512, "limit": 7.0}}
+
+
 def _mogisun_layer(kind, moe):
     if kind == "attention":
         mixer = {"heads": 8, "kv_heads": 2, "dim": 64, "vdim": 64, "scale": 0.125, "q_temp": {"coef": 0.2, "every": 512}}
@@ -98,6 +114,15 @@ PRESETS = {
                    _famepel_layer({"type": "mamba2", "mixer": {"conv": 4, "groups": 2, "heads": 8, "norm_groups": 2,
                                                                  "state": 64, "vdim": 64}}),
                    _famepel_layer(dict(_FAMEPEL_LATENT, mixer=dict(_FAMEPEL_LATENT["mixer"], kv_from=2)))],
+    },
+    # a small model of the Tadinex design: three delta-rule layers after every layer of the two mixers side by side,
+    # a dense feed-forward first, routed experts after it
+    "tadinex-small": {
+        "architecture": "Tadinex", "vocab": 4096, "width": 512, "norm": {"eps": 1e-6}, "embedding": {"scale": 8.0},
+        "residual_mult": 0.8,
+        "layers": [_tadinex_layer("parallel", {"kind": "dense", "ff": 1536}), _tadinex_layer("delta", _TADINEX_EXPERTS),
+                   _tadinex_layer("delta", _TADINEX_EXPERTS), _tadinex_layer("delta", _TADINEX_EXPERTS),
+                   _tadinex_layer("parallel", _TADINEX_EXPERTS), _tadinex_layer("delta", _TADINEX_EXPERTS)],
     },
     "tiny-a": {
         "architectures": ["LlamaForCausalLM"], "model_type": "llama",

@@ -72,13 +72,15 @@ struct Epilogue {
     ResidualOut res;
     RowScale scale;
     int activation;   // EPI_ACT: which (SiaActivation)
+    int glu;          // EPI_SWIGLU: which gated activation (SiaGlu; 0 is silu(gate) * up)
+    float limit;      // EPI_SWIGLU: the clamp of the gated activations that have one
 };
 
 // RB: blocks of bh rows of W per workgroup; WAVES: 8 or 16 waves that split K.
 //   EPI_STORE:   row block rb holds bh rows of W and gives as many columns of Y (TOut)
 //   EPI_ACT:     as EPI_STORE, with an activation without a gate applied to the float sums, rounded once
 //   EPI_SWIGLU:  W = [gate; up] of N rows each; the first RB / 2 row blocks are gate rows, the others the up rows of
-//                the same columns: Y = silu(gate) * up, in float, rounded once
+//                the same columns: Y = silu(gate) * up (or another gated activation of common.h), in float, rounded once
 //   EPI_ROPE:    RB = 2, W = [q heads | k heads | v heads] of head_dim rows each; a workgroup owns 16 columns of
 //                the first half of a head and the 16 that the rotation pairs them with (head_dim / 2 further).
 //                q and k are rotated in float on the float sums (one rounding; the rotation kernel rotates the
@@ -306,7 +308,8 @@ __global__ __launch_bounds__(WAVES* SIA_WAVE) void gemm_skinny_kernel(const bf16
             float gate = total(j, m, n), up = total(UNIT_BLOCKS + j, m, n);
             gate *= rs;
             up *= rs;
-            *y = from_float<TOut>(gate / (1.f + expf(-gate)) * up);
+            *y = from_float<TOut>(ep.glu == SIA_GLU_SILU ? gate / (1.f + expf(-gate)) * up
+                                                         : gated_activation(gate, up, ep.glu, ep.limit));
         } else if (EPI == EPI_ACT) {
             *y = from_float<TOut>(activate(total(j, m, n) * rs, ep.activation));
         } else {
@@ -461,12 +464,17 @@ SIA_EXPORT int sia_gemm_skinny_tiled(const void* X, const void* W_tiled, void* Y
 // Y[M, I] = silu(X Wg^T) * (X Wu^T) for W = [Wg; Wu] of 2 I rows.  Needs M <= 16, K % 64 == 0.
 // With `partials` (else null) X is a `scaled` matrix of sia_gemm_skinny_residual and the rows are divided by their
 // root mean square first.
-SIA_EXPORT int sia_gemm_skinny_swiglu(const void* X, const void* W, void* Y, int M, int inter, int K,
-                                      const float* partials, int n_partials, float eps, hipStream_t stream) {
+// glu, limit: another gated activation than silu(gate) * up (SiaGlu of common.h).
+SIA_EXPORT int sia_gemm_skinny_glu(const void* X, const void* W, void* Y, int M, int inter, int K,
+                                   const float* partials, int n_partials, float eps, int glu, float limit,
+                                   hipStream_t stream) {
     if (M <= 0 || inter <= 0) return 0;
-    if (M > 16 || K % 64 || K <= 0 || (partials && n_partials <= 0)) return SIA_BAD_ARGUMENT;
+    if (M > 16 || K % 64 || K <= 0 || (partials && n_partials <= 0) || (glu != SIA_GLU_SILU && glu != SIA_GLU_CLAMPED))
+        return SIA_BAD_ARGUMENT;
     Epilogue ep{};
     ep.scale = RowScale{partials, n_partials, eps};
+    ep.glu = glu;
+    ep.limit = limit;
     const Cut cut = cheapest(inter, 2, {2, 1});
 #define LAUNCH(RB, WAVES, SCALED)                                                                                  \
     hipLaunchKernelGGL((gemm_skinny_kernel<bf16_t, RB, WAVES, EPI_SWIGLU, SCALED>), dim3(cut.grid),              \
@@ -482,6 +490,11 @@ SIA_EXPORT int sia_gemm_skinny_swiglu(const void* X, const void* W, void* Y, int
         LAUNCH(2, 8, false);
 #undef LAUNCH
     return SIA_LAUNCH_CHECK();
+}
+
+SIA_EXPORT int sia_gemm_skinny_swiglu(const void* X, const void* W, void* Y, int M, int inter, int K,
+                                      const float* partials, int n_partials, float eps, hipStream_t stream) {
+    return sia_gemm_skinny_glu(X, W, Y, M, inter, K, partials, n_partials, eps, SIA_GLU_SILU, 0.f, stream);
 }
 
 // The q/k/v product of single-token steps with the rotation and the cache write in its epilogue:

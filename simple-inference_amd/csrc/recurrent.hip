@@ -856,6 +856,162 @@ __global__ __launch_bounds__(512) void delta_rule_kernel(
     }
 }
 
+// The same walk for a prompt's step in bfloat16, laid out as the linear attention's walk above: the 16 lanes of one
+// row of a wave share C columns of the state, lane r keeping rows r * ROWS .. r * ROWS + ROWS - 1 of each, so that what
+// a lane reads of q and k from LDS serves all its columns and the two sums of a token (S^T k before the write, S^T q
+// after it) are exchanges inside the vector unit.  q and k lie in LDS as floats so that the 16 lanes' 16-byte pieces
+// of a read are one contiguous run; rows beyond D are zero.  Blocks of 32 tokens; a block's unit norms, write
+// strengths and decays are taken in LDS before it is walked, and its outputs leave together.
+#define DELTA_WALK_TOKENS 32
+#define DELTA_WALK_THREADS 256
+template <int ROWS, int C>
+__global__ __launch_bounds__(DELTA_WALK_THREADS) void delta_walk_kernel(
+    const bf16_t* __restrict__ qkv, int qkv_stride, const bf16_t* __restrict__ proj, int proj_stride, int b_col,
+    int a_col, const float* __restrict__ a_log, const float* __restrict__ dt_bias, float* __restrict__ state,
+    long long state_stride, const int* __restrict__ cu_q, const int* __restrict__ slots, float* __restrict__ raw_out,
+    int n_heads, int n_kv, int D, int Dv) {
+    extern __shared__ float lds[];
+    constexpr int TB = DELTA_WALK_TOKENS, threads = DELTA_WALK_THREADS;
+    constexpr int slice = threads / 16 * C;      // columns a workgroup
+    constexpr int Dp = 16 * ROWS;
+    const int seq = blockIdx.x, head = blockIdx.y, tid = threadIdx.x;
+    const int j0 = blockIdx.z * slice;
+    const int first = cu_q[seq], last = cu_q[seq + 1];
+    if (first >= last) return;
+    float* q_s = lds;               // [TB][Dp], row d = r * ROWS + i at (i / 4) * 64 + r * 4 + i % 4
+    float* k_s = q_s + TB * Dp;
+    float* v_s = k_s + TB * Dp;     // [TB][slice]
+    float* o_s = v_s + TB * slice;  // [TB][slice]
+    float* be_s = o_s + TB * slice; // [TB]
+    float* de_s = be_s + TB;        // [TB]
+    auto place = [](int d) { const int r = d / ROWS, i = d % ROWS; return (i / 4) * 64 + r * 4 + i % 4; };
+    for (int i = tid; i < 2 * TB * Dp; i += threads) lds[i] = 0.f;
+    const int jl = (tid / 16) * C, r = tid % 16;
+    float* S_mem = state + (size_t)slots[seq] * state_stride + (size_t)head * D * Dv;
+    float S[C][ROWS];
+#pragma unroll
+    for (int c = 0; c < C; ++c)
+#pragma unroll
+        for (int i = 0; i < ROWS; ++i) {
+            const int d = r * ROWS + i, j = j0 + jl + c;
+            S[c][i] = (j < Dv && d < D) ? S_mem[(size_t)d * Dv + j] : 0.f;
+        }
+    const int wave = tid / SIA_WAVE, lane = tid % SIA_WAVE;
+    const int kv_head = head / (n_heads / n_kv);
+    const int q_col = kv_head * D, k_col = n_kv * D + kv_head * D, v_col = 2 * n_kv * D + head * Dv;
+    const float rate = expf(a_log[head]), bias = dt_bias ? dt_bias[head] : 0.f;
+    const float q_scale = rsqrtf((float)D);
+    __syncthreads();
+    for (int t0 = first; t0 < last; t0 += TB) {
+        const int nt = min(TB, last - t0);
+        for (int idx = tid; idx < nt * D; idx += threads) {
+            const int t = idx / D, d = idx % D;
+            const bf16_t* row = qkv + (size_t)(t0 + t) * qkv_stride;
+            q_s[t * Dp + place(d)] = bf16_to_float(row[q_col + d]);
+            k_s[t * Dp + place(d)] = bf16_to_float(row[k_col + d]);
+        }
+        for (int idx = tid; idx < nt * slice; idx += threads) {
+            const int t = idx / slice, c = idx % slice;
+            v_s[idx] = j0 + c < Dv ? bf16_to_float(qkv[(size_t)(t0 + t) * qkv_stride + v_col + j0 + c]) : 0.f;
+        }
+        if (tid < nt) {
+            const bf16_t* row = proj + (size_t)(t0 + tid) * proj_stride;
+            const float zb = bf16_to_float(row[b_col + head]), za = bf16_to_float(row[a_col + head]) + bias;
+            be_s[tid] = 1.f / (1.f + expf(-zb));
+            de_s[tid] = expf(-rate * (fmaxf(za, 0.f) + log1pf(expf(-fabsf(za)))));
+        }
+        __syncthreads();
+        for (int t = wave; t < nt; t += threads / SIA_WAVE) {      // unit vectors, a wave a token (the padding is zero)
+            float sq = 0.f, sk = 0.f;
+            for (int c = lane; c < Dp; c += SIA_WAVE) {
+                sq += q_s[t * Dp + c] * q_s[t * Dp + c];
+                sk += k_s[t * Dp + c] * k_s[t * Dp + c];
+            }
+            const float iq = rsqrtf(wave_sum(sq) + 1e-6f) * q_scale, ik = rsqrtf(wave_sum(sk) + 1e-6f);
+            for (int c = lane; c < Dp; c += SIA_WAVE) {
+                q_s[t * Dp + c] *= iq;
+                k_s[t * Dp + c] *= ik;
+            }
+        }
+        __syncthreads();
+        float4 qn[ROWS / 4], kn[ROWS / 4];
+        auto fetch = [&](int t) {
+#pragma unroll
+            for (int i = 0; i < ROWS / 4; ++i) {
+                const int at = t * Dp + i * 64 + r * 4;
+                qn[i] = *reinterpret_cast<const float4*>(q_s + at);
+                kn[i] = *reinterpret_cast<const float4*>(k_s + at);
+            }
+        };
+        fetch(0);
+        for (int t = 0; t < nt; ++t) {
+            float4 qv[ROWS / 4], kv[ROWS / 4];
+            float vv[C];
+#pragma unroll
+            for (int i = 0; i < ROWS / 4; ++i) { qv[i] = qn[i]; kv[i] = kn[i]; }
+#pragma unroll
+            for (int c = 0; c < C; ++c) vv[c] = v_s[t * slice + jl + c];
+            const float g = de_s[t], b = be_s[t];
+            fetch(min(t + 1, TB - 1));
+            float kept[C];
+#pragma unroll
+            for (int c = 0; c < C; ++c) {
+                float acc = 0.f;
+#pragma unroll
+                for (int i = 0; i < ROWS / 4; ++i) {
+                    S[c][4 * i] *= g;
+                    S[c][4 * i + 1] *= g;
+                    S[c][4 * i + 2] *= g;
+                    S[c][4 * i + 3] *= g;
+                    acc += kv[i].x * S[c][4 * i];
+                    acc += kv[i].y * S[c][4 * i + 1];
+                    acc += kv[i].z * S[c][4 * i + 2];
+                    acc += kv[i].w * S[c][4 * i + 3];
+                }
+                kept[c] = acc;
+            }
+#pragma unroll
+            for (int c = 0; c < C; ++c) kept[c] = row16_sum(kept[c]);
+            float out[C];
+#pragma unroll
+            for (int c = 0; c < C; ++c) {
+                const float u = b * (vv[c] - kept[c]);
+                float acc = 0.f;
+#pragma unroll
+                for (int i = 0; i < ROWS / 4; ++i) {
+                    S[c][4 * i] += kv[i].x * u;
+                    S[c][4 * i + 1] += kv[i].y * u;
+                    S[c][4 * i + 2] += kv[i].z * u;
+                    S[c][4 * i + 3] += kv[i].w * u;
+                    acc += qv[i].x * S[c][4 * i];
+                    acc += qv[i].y * S[c][4 * i + 1];
+                    acc += qv[i].z * S[c][4 * i + 2];
+                    acc += qv[i].w * S[c][4 * i + 3];
+                }
+                out[c] = acc;
+            }
+#pragma unroll
+            for (int c = 0; c < C; ++c) {
+                out[c] = row16_sum(out[c]);
+                if (r == 0) o_s[t * slice + jl + c] = out[c];
+            }
+        }
+        __syncthreads();
+        for (int idx = tid; idx < nt * slice; idx += threads)
+            if (j0 + idx % slice < Dv)
+                raw_out[((size_t)(t0 + idx / slice) * n_heads + head) * Dv + j0 + idx % slice] = o_s[idx];
+        // (the next block's staging touches q_s, k_s, v_s and the gates, which nobody reads any more; o_s is written
+        // again only behind two more barriers)
+    }
+#pragma unroll
+    for (int c = 0; c < C; ++c)
+#pragma unroll
+        for (int i = 0; i < ROWS; ++i) {
+            const int d = r * ROWS + i, j = j0 + jl + c;
+            if (j < Dv && d < D) S_mem[(size_t)d * Dv + j] = S[c][i];
+        }
+}
+
 // floats of workspace: the raw outputs [tokens, heads, Dv]
 SIA_EXPORT long long sia_delta_rule_workspace(int n_tokens, int n_heads, int Dv) {
     return (long long)n_tokens * n_heads * Dv;
@@ -892,6 +1048,25 @@ SIA_EXPORT int sia_delta_rule(const void* qkv, int qkv_stride, const void* proj,
     while (TB > 1 && bytes(TB) > 60 * 1024) TB /= 2;
     if (bytes(TB) > 60 * 1024) return SIA_BAD_ARGUMENT;
     dim3 grid(n_seqs, n_heads, (Dv + slice - 1) / slice), block(threads), fgrid(n_tokens, n_heads), fblock(SIA_WAVE);
+    // a prompt's step in bfloat16: the walk whose lanes share columns, where its rows fit a lane's registers and LDS
+    constexpr int w_cols = 2, w_slice = DELTA_WALK_THREADS / 16 * w_cols;
+    const int w_rows = (D + 15) / 16;
+    const int w_rows_t = w_rows <= 4 ? 4 : w_rows <= 8 ? 8 : w_rows <= 16 ? 16 : 32;
+    const size_t w_lds = (size_t)(DELTA_WALK_TOKENS * (2 * 16 * w_rows_t + 2 * w_slice + 2)) * sizeof(float);
+    if (max_q_len > 1 && dtype == SIA_BF16 && w_rows_t <= 16 && w_lds <= 60 * 1024) {
+        dim3 wgrid(n_seqs, n_heads, (Dv + w_slice - 1) / w_slice), wblock(DELTA_WALK_THREADS);
+#define WALK(ROWS)                                                                                                   \
+    hipLaunchKernelGGL((delta_walk_kernel<ROWS, w_cols>), wgrid, wblock, w_lds, stream, (const bf16_t*)qkv,          \
+                       qkv_stride, (const bf16_t*)proj, proj_stride, b_col, a_col, a_log, dt_bias, state,            \
+                       state_stride, cu_q, slots, workspace, n_heads, n_kv, D, Dv)
+        if (w_rows_t == 4) WALK(4);
+        else if (w_rows_t == 8) WALK(8);
+        else WALK(16);
+#undef WALK
+        hipLaunchKernelGGL(gla_finish_kernel<bf16_t>, fgrid, fblock, 0, stream, workspace, (const bf16_t*)proj,
+                           proj_stride, g_col, norm_w, (bf16_t*)out, n_heads, Dv, eps);
+        return SIA_LAUNCH_CHECK();
+    }
 #define LAUNCH(T, ROWS)                                                                                              \
     hipLaunchKernelGGL((delta_rule_kernel<T, ROWS>), grid, block, bytes(TB), stream, (const T*)qkv, qkv_stride,      \
                        (const T*)proj, proj_stride, b_col, a_col, a_log, dt_bias, state, state_stride, cu_q, slots,   \

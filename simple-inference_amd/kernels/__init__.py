@@ -105,6 +105,7 @@ _SIGNATURES = {
     "sia_add_rmsnorm_scaled": [_c_ptr, _c_ptr, _c_float, _c_ptr, _c_float, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_float,
                                _c_int, _c_ptr],
     "sia_scaled_sum": [_c_ptr, _c_float, _c_ptr, _c_float, _c_ptr, _c_ll, _c_int, _c_ptr],
+    "sia_gemm_skinny_glu": [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr, _c_int, _c_float, _c_int, _c_float, _c_ptr],
     "sia_glu": [_c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_float, _c_int, _c_ptr],
     "sia_qk_prepare_ex": [_c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_float, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int,
                           _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr,
@@ -1000,6 +1001,15 @@ class HipKernels:
         two_i = w_gate_up.shape[0]
         if activation is not None:
             glu, limit = self._glu(activation)
+            if (self.use_skinny_gemm and x.dtype == torch.bfloat16 and w_gate_up.dtype == torch.bfloat16
+                    and M <= self._skinny_rows and two_i % 2 == 0 and K % 64 == 0 and w_gate_up.shape[1] == K):
+                rows, partials, n_partials, eps = self._scaled(x)      # few rows: the activation inside the product
+                self._want(rows, "gated linear input")
+                y = torch.empty((M, two_i // 2), dtype=torch.bfloat16, device=rows.device)
+                self._check(self.core.sia_gemm_skinny_glu(_ptr(rows), _ptr(w_gate_up), _ptr(y), M, two_i // 2, K,
+                                                          _ptr(partials), n_partials, eps, glu, limit, self._stream()),
+                            "gemm_skinny_glu")
+                return y
             gu = self.linear(x, w_gate_up)
             if gu.dtype not in _DT or two_i % 2:
                 raise KernelError(f"a gated activation takes [tokens, 2 * intermediate] rows, got {gu.dtype} {tuple(gu.shape)}")
