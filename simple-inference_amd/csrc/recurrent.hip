@@ -762,7 +762,9 @@ __global__ __launch_bounds__(512) void delta_rule_kernel(
     const T* __restrict__ qkv, int qkv_stride, const T* __restrict__ proj, int proj_stride, int b_col, int a_col,
     const float* __restrict__ a_log, const float* __restrict__ dt_bias, float* __restrict__ state,
     long long state_stride, const int* __restrict__ cu_q, const int* __restrict__ slots, float* __restrict__ raw_out,
-    int n_heads, int n_kv, int D, int Dv, int R, int block_tokens, int slice) {
+    int n_heads, int n_kv, int D, int Dv, int R, int block_tokens, int slice, int g_col,
+    const float* __restrict__ norm_w, T* __restrict__ out, float eps) {
+    // raw_out absent: the workgroup owns all of the head's columns (slice == Dv) and norms and gates its outputs itself
     extern __shared__ float lds[];
     const int seq = blockIdx.x, head = blockIdx.y, tid = threadIdx.x;
     const int j0 = blockIdx.z * slice;
@@ -774,6 +776,7 @@ __global__ __launch_bounds__(512) void delta_rule_kernel(
     float* v_s = k_s + TB * D;         // [TB][slice]
     float* be_s = v_s + TB * slice;    // [TB]
     float* de_s = be_s + TB;           // [TB]
+    float* o_s = de_s + TB;            // [TB][slice], without raw_out only
     const int j = j0 + tid / R, r = tid % R;
     const bool owns = tid / R < slice && j < Dv;
     float* S_mem = state + (size_t)slots[seq] * state_stride + (size_t)head * D * Dv;
@@ -845,7 +848,23 @@ __global__ __launch_bounds__(512) void delta_rule_kernel(
                 }
             }
             for (int o = R / 2; o > 0; o >>= 1) acc += __shfl_xor(acc, o, SIA_WAVE);
-            if (owns && r == 0) raw_out[((size_t)(t0 + t) * n_heads + head) * Dv + j] = acc;
+            if (owns && r == 0) {
+                if (raw_out) raw_out[((size_t)(t0 + t) * n_heads + head) * Dv + j] = acc;
+                else o_s[t * slice + (j - j0)] = acc;
+            }
+        }
+        __syncthreads();
+        if (raw_out) continue;   // uniform: the norm is another kernel's
+        for (int t = wave; t < nt; t += n_waves) {
+            float ss = 0.f;
+            for (int c = lane; c < Dv; c += SIA_WAVE) ss += o_s[t * slice + c] * o_s[t * slice + c];
+            const float inv = rsqrtf(wave_sum(ss) / (float)Dv + eps);
+            const T* g_row = proj + (size_t)(t0 + t) * proj_stride + g_col + head * Dv;
+            T* dst = out + ((size_t)(t0 + t) * n_heads + head) * Dv;
+            for (int c = lane; c < Dv; c += SIA_WAVE) {
+                const float z = to_float(g_row[c]);
+                dst[c] = from_float<T>(o_s[t * slice + c] * inv * norm_w[c] * (z / (1.f + expf(-z))));
+            }
         }
         __syncthreads();
     }
@@ -1044,9 +1063,12 @@ SIA_EXPORT int sia_delta_rule(const void* qkv, int qkv_stride, const void* proj,
     if (rows > 128) return SIA_BAD_ARGUMENT;
     const int threads = ((slice * R + SIA_WAVE - 1) / SIA_WAVE) * SIA_WAVE;
     int TB = max_q_len >= 16 ? 16 : (max_q_len >= 4 ? 4 : 1);
-    auto bytes = [&](int tb) { return (size_t)tb * (2 * D + slice + 2) * sizeof(float); };
+    // a workgroup that owns a whole head norms and gates its outputs itself (a decode step: one launch less)
+    const bool whole = slice == Dv;
+    auto bytes = [&](int tb) { return (size_t)tb * (2 * D + (whole ? 2 : 1) * slice + 2) * sizeof(float); };
     while (TB > 1 && bytes(TB) > 60 * 1024) TB /= 2;
     if (bytes(TB) > 60 * 1024) return SIA_BAD_ARGUMENT;
+    float* raw = whole ? nullptr : workspace;
     dim3 grid(n_seqs, n_heads, (Dv + slice - 1) / slice), block(threads), fgrid(n_tokens, n_heads), fblock(SIA_WAVE);
     // a prompt's step in bfloat16: the walk whose lanes share columns, where its rows fit a lane's registers and LDS
     constexpr int w_cols = 2, w_slice = DELTA_WALK_THREADS / 16 * w_cols;
@@ -1070,7 +1092,7 @@ SIA_EXPORT int sia_delta_rule(const void* qkv, int qkv_stride, const void* proj,
 #define LAUNCH(T, ROWS)                                                                                              \
     hipLaunchKernelGGL((delta_rule_kernel<T, ROWS>), grid, block, bytes(TB), stream, (const T*)qkv, qkv_stride,      \
                        (const T*)proj, proj_stride, b_col, a_col, a_log, dt_bias, state, state_stride, cu_q, slots,   \
-                       workspace, n_heads, n_kv, D, Dv, R, TB, slice)
+                       raw, n_heads, n_kv, D, Dv, R, TB, slice, g_col, norm_w, (T*)out, eps)
 #define RUN(T)                                                                                                       \
     do {                                                                                                             \
         if (rows <= 4) LAUNCH(T, 4);                                                                                 \
@@ -1079,8 +1101,9 @@ SIA_EXPORT int sia_delta_rule(const void* qkv, int qkv_stride, const void* proj,
         else if (rows <= 32) LAUNCH(T, 32);                                                                          \
         else if (rows <= 64) LAUNCH(T, 64);                                                                          \
         else LAUNCH(T, 128);                                                                                         \
-        hipLaunchKernelGGL(gla_finish_kernel<T>, fgrid, fblock, 0, stream, workspace, (const T*)proj, proj_stride,   \
-                           g_col, norm_w, (T*)out, n_heads, Dv, eps);                                                \
+        if (raw)                                                                                                     \
+            hipLaunchKernelGGL(gla_finish_kernel<T>, fgrid, fblock, 0, stream, workspace, (const T*)proj,            \
+                               proj_stride, g_col, norm_w, (T*)out, n_heads, Dv, eps);                               \
     } while (0)
     if (dtype == SIA_F32) RUN(float);
     else if (dtype == SIA_BF16) RUN(bf16_t);

@@ -303,7 +303,7 @@ def window_part(k, dev, dtype, g, hidden, H, G, D, window, dims, scaling, scale=
 @pytest.mark.parametrize("backend", BACKENDS)
 @pytest.mark.parametrize("H,G,D,window,dims,scaling,page", [
     (4, 2, 16, 11, 8, (4.0, 64, 16.0, 2.0), 8), (2, 2, 24, 40, 24, None, 16), (4, 1, 64, 24, 32, (16.0, 128, 32.0, 1.0), 16),
-    (5, 5, 12, 7, 4, (2.0, 40, 8.0, 1.0), 16), (1, 1, 32, 1, 16, None, 16), (6, 2, 96, 33, 48, (2.0, 256, 32.0, 1.0), 16)])
+    (5, 5, 12, 7, 4, (2.0, 40, 8.0, 1.0), 16), (1, 1, 32, 1, 16, None, 16), (6, 2, 80, 33, 40, (3.0, 256, 24.0, 1.0), 16)])
 def test_window_attention_whose_values_are_its_keys_as_projected(backend, H, G, D, window, dims, scaling, page):
     """A prompt in portions and decoded tokens (positions that pass the window and pages' borders) against the plain
     function over the whole sequence: values that are the keys before norm and rotation, the sink, the window."""
