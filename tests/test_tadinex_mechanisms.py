@@ -52,7 +52,7 @@ def test_scaled_terms_go_into_the_residual_inside_the_norm(backend, width):
 def test_exact_gelu_and_the_clamped_gate(backend):
     k, dev, dtype, tol = setup(backend)
     g = torch.Generator().manual_seed(3)
-    for n, width, inter in ((5, 64, 40), (33, 128, 72)):
+    for n, width, inter in ((5, 64, 40), (33, 128, 72), (19, 64, 27)):
         x, x64 = lowered(rnd(g, n, width), dtype, dev)
         w, w64 = lowered(rnd(g, 2 * inter, width, std=0.4), dtype, dev)
         close(k.activated_linear(x, w, "gelu"), plain.gelu_erf(x64 @ w64.T), tol)
